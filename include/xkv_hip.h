@@ -1,0 +1,151 @@
+/* xkv_hip.h - C ABI of libxkv_hip.so: MI355X (gfx950) kernels of the xKV compressed-KV decode path.
+ *
+ * The reference project is pure Python + Triton; the "FFI" each entry point replaces is
+ * therefore a Triton kernel launch (`kernel[grid](...)`) inside one of its Python wrappers.
+ * Each prototype cites that launch (paths relative to the reference repository).
+ *
+ * Conventions
+ *   - plain pointers, 32/64-bit integers and floats only; no torch / pybind types.
+ *   - every pointer is DEVICE memory unless named host_*; the library never allocates,
+ *     frees or keeps state between calls (workspaces are caller-owned).
+ *   - all launches go to `stream` (a hipStream_t passed as void*) and return without
+ *     synchronising.  Return value: XKV_OK, a negative XKV_E* argument error detected on the
+ *     host before any launch, or a positive hipError_t from the launch.
+ *   - strides are in ELEMENTS.  The innermost (feature) axis of every 16-bit operand is
+ *     unit-stride and every row start is 16-byte aligned (strides multiple of 8 elements).
+ *   - `dtype` is the 16-bit operand type of q / A / B / K / V (XKV_F16 or XKV_BF16);
+ *     accumulation is always fp32.
+ *   - split arithmetic (which tokens split i of a sequence covers, which splits are live) is
+ *     the reference's, flash_decoding/gqa.py:95-99 and :273-281, bit for bit, with the
+ *     sequence length taken from kv_lens[b] when kv_lens != NULL (ragged batch) else kv_len.
+ */
+#ifndef XKV_HIP_H
+#define XKV_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XKV_ABI_VERSION 1
+
+enum { XKV_F16 = 0, XKV_BF16 = 1, XKV_F32 = 2 };
+
+enum {
+  XKV_OK = 0,
+  XKV_EINVAL = -1,      /* null pointer / non-positive size */
+  XKV_EUNSUPPORTED = -2,/* shape outside the built envelope (see each function) */
+  XKV_EALIGN = -3,      /* stride or pointer not 16-byte aligned */
+  XKV_EDTYPE = -4
+};
+
+int xkv_abi_version(void);
+const char* xkv_error_string(int code);
+
+/* RoPE tables: sin[l, j] / cos[l, j] of angle float(start + l) * inv_freq[j], l < seqlen, j < half_dim,
+ * written as out_dtype (XKV_F32 / XKV_F16 / XKV_BF16), row stride = half_dim.
+ * Replaces _rotary_sin_cos_kernel_multi[grid] at flash_recontruction/rope/sin_cos.py:92-97
+ * (angles follow the eager closed form of rope/rope_ref.py:3-9: fp32 pos * fp32 inv_freq). */
+int xkv_rope_table(void* sin_out, void* cos_out, const float* inv_freq, int64_t seqlen, int64_t start,
+                   int half_dim, int out_dtype, void* stream);
+
+/* Absorb the query into the per-kv-head factor: qt[b, h, rho] = sum_d q[b, h, d] * B[b, h / G, rho, d]
+ * as a 16-bit high part `qt_hi` and (optional, may be NULL) residual `qt_lo` so that hi + lo carries
+ * ~16 mantissa bits.  q is [batch, hq, d] contiguous.  qt_* are [batch, hq, rank] contiguous.
+ * Replaces the host-side torch.matmul(q_nope, kv_B_nope.transpose(1, 2)) at
+ * flash_decoding/mla2/mla_flash_decoding.py:81-82 and is what makes the no-PE score scan a GEMV
+ * over A (the eager form attention.py:312-318) instead of the per-tile reconstruction of
+ * flash_recontruction/qAB_no_pe/v1.py:53-74.   d <= 256, d % 8 == 0. */
+int xkv_absorb_q(const void* q, const void* B, void* qt_hi, void* qt_lo,
+                 int batch, int hq, int hkv, int d, int rank,
+                 int64_t stride_B_b, int64_t stride_B_h, int64_t stride_B_r,
+                 int dtype, void* stream);
+
+/* Operand descriptors of the generic split-K stage 1. */
+typedef struct {
+  const void* ptr;     /* [batch, kv_len, heads?, dim]; NULL = absent                      */
+  int64_t stride_b;    /* batch stride                                                     */
+  int64_t stride_l;    /* token stride                                                     */
+  int64_t stride_h;    /* kv-head stride (0 when one latent serves every head)             */
+  int dim;             /* feature width                                                    */
+} xkv_kv_operand;
+
+typedef struct {
+  const void* ptr;     /* [batch, hq, dim] contiguous; NULL = absent                       */
+  int dim;
+} xkv_q_operand;
+
+/* Split-K flash-decoding stage 1 over "latent-like" operands (plain dot-product scores):
+ *
+ *   s[b, h, l]   = sm_scale * ( qn[b,h,:] . C[b,l,kvh(h),:]  (+ qn_lo . C)  (+ qr[b,h,:] . R[b,l,kvh(h),:]) )
+ *   per live split i of sequence b (tokens [start,end)):
+ *     m = max_l s ; den = sum_l exp(s - m) ; partial[b,h,i,:] = sum_l exp(s-m) V[b,l,kvh(h),:] / den ;
+ *     lse[b,h,i] = m + log(den)
+ *
+ * kvh(h) = h / (hq / n_kv_groups).  With n_kv_groups == 1 every head shares one latent row
+ * (xKV no-PE after xkv_absorb_q: C = k_A, V = v_A; MLA: C = V = c_kv, R = k_pe).  With
+ * n_kv_groups == hkv it is plain GQA (C = K, V = V) or a mix (C = K, V = v_A with stride_h 0).
+ * If V.ptr == C.ptr with equal strides and dim the tile is loaded once.
+ * If scores_out != NULL the kernel ONLY writes scores (scaled) as [batch, hq, kv_len] in
+ * scores_dtype and skips softmax/PV (qAB no-PE form).
+ * Dead splits write nothing.  partial is [batch, hq, max_splits, V.dim] fp32, lse [batch, hq, max_splits] fp32.
+ * Envelope: heads per kv group <= 32; C.dim % 32 == 0, <= 1024; R.dim % 32 == 0, <= 128;
+ *           V.dim % 64 == 0, <= 512.
+ * Replaces _fwd_grouped_kernel_stage1[grid] at flash_decoding/gqa.py:205-237,
+ * flash_decoding/mla.py (same launcher, :243-283), flash_decoding/mla2/stage1.py:213-249,
+ * flash_recontruction/fused_attention/no_pe/v1.py:227-262 (and v2.py / v1_k_only.py twins) and,
+ * in scores_out mode, _qAB_fwd[grid] at flash_recontruction/qAB_no_pe/v1.py:123-132 (v2.py:117-126). */
+int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_operand qr,
+                      xkv_kv_operand C, xkv_kv_operand R, xkv_kv_operand V,
+                      float* partial, float* lse,
+                      void* scores_out, int scores_dtype,
+                      const int32_t* num_kv_splits, const int32_t* kv_lens,
+                      int batch, int hq, int n_kv_groups, int kv_len, int max_splits,
+                      float sm_scale, float logit_cap, int dtype, void* stream);
+
+/* Split-K stage 1 with fused key reconstruction and RoPE:
+ *
+ *   K[b,kh,l,:]  = kA[b,l,:] @ kB[b,kh,:,:]                      (rank x 128, fp32 accumulate)
+ *   K'           = rotate-half RoPE of K at position pos_offset + l, angle float(pos) * inv_freq[j]
+ *                  (or, if sin_cos != NULL, sin = sin_cos[l, j], cos = sin_cos[l, 64 + j], a
+ *                  [kv_len, 128] table of the operand dtype, row stride sc_stride_l)
+ *   s[b,h,l]     = sm_scale * q_pe[b,h,:] . K'[b,h/G,l,:]        (K' rounded to the operand dtype)
+ *
+ * then either scores_out (as above) or the split softmax with V = vA (rank-space partials
+ * [batch, hq, max_splits, vA.dim]).  rope == 0 skips the rotation (pure reconstruction).
+ * Envelope: head_dim == 128, G = hq/hkv <= 16, rank % 32 == 0, rank <= 512, vA.dim % 64 == 0 <= 512.
+ * Replaces _qAB_fwd[grid] at flash_recontruction/qAB/v1.py:135-145 (v3.py / v4.py / ref.py twins) and
+ * _qAB_fwd_precomp[grid] at qAB/v2.py:170-186 in scores_out mode; the fused form has no single
+ * reference launch - it composes that reconstruction with the stage 1 of
+ * fused_attention/no_pe/v1.py:227-262. */
+int xkv_recon_stage1(const void* q_pe, xkv_kv_operand kA, const void* kB,
+                     int64_t stride_kB_b, int64_t stride_kB_h, int64_t stride_kB_r,
+                     xkv_kv_operand vA,
+                     float* partial, float* lse,
+                     void* scores_out, int scores_dtype,
+                     const int32_t* num_kv_splits, const int32_t* kv_lens,
+                     int batch, int hq, int hkv, int kv_len, int max_splits,
+                     float sm_scale, int rope, const float* inv_freq, int64_t pos_offset,
+                     const void* sin_cos, int64_t sc_stride_l,
+                     int dtype, void* stream);
+
+/* Stage 2: LSE-weighted merge of the live splits in increasing split id,
+ *   out[b,h,:] = sum_i w_i partial[b,h,i,:] / sum_i w_i ,  w_i = exp(lse_i - max lse),
+ * optionally followed by the value up-projection out[b,h,:] = merged[b,h,:] @ vB[b, h/G, :, :]
+ * (vB == NULL: none; then out width = dv).  out is [batch, hq, out_dim] with strides
+ * (stride_o_b, stride_o_h), written as out_dtype.
+ * Replaces _fwd_kernel_stage2[grid] at flash_decoding/gqa.py:322-337 (mla.py, mla2/stage2.py:117-135,
+ * fused_attention/no_pe/v1.py:345-362 twins) and the torch.matmul with v_B_buffer at
+ * fused_attention/no_pe/v2.py:468-471 / v1.py:458-460.   dv <= 512; d_out <= 256. */
+int xkv_merge_stage2(const float* partial, const float* lse, void* out,
+                     const void* vB, int64_t stride_vB_b, int64_t stride_vB_h, int64_t stride_vB_r,
+                     int d_out, int vB_dtype,
+                     const int32_t* num_kv_splits, const int32_t* kv_lens,
+                     int batch, int hq, int hkv, int kv_len, int max_splits, int dv,
+                     int64_t stride_o_b, int64_t stride_o_h, int out_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XKV_HIP_H */

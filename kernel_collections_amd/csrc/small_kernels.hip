@@ -1,0 +1,221 @@
+// RoPE table, query absorption and the stage-2 merge: the small kernels around the scans.
+#include "xkv_common.h"
+
+namespace xkv {
+
+// ----------------------------------------------------------------------------------------------
+// RoPE table.  angle = float(pos) * inv_freq[j] in fp32 (one rounding), then sincosf with full
+// range reduction - the eager closed form of the reference (rope/rope_ref.py:3-9), not the
+// fast-math pow/sin/cos of its Triton table kernel.
+// ----------------------------------------------------------------------------------------------
+template <typename O>
+__global__ void rope_table_kernel(O* __restrict__ sin_out, O* __restrict__ cos_out,
+                                  const float* __restrict__ inv_freq, int64_t seqlen, int64_t start,
+                                  int half_dim) {
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= seqlen * half_dim) return;
+  int j = (int)(idx % half_dim);
+  int64_t l = idx / half_dim;
+  float ang = (float)(start + l) * inv_freq[j];
+  float s, c;
+  sincosf(ang, &s, &c);
+  sin_out[idx] = (O)s;
+  cos_out[idx] = (O)c;
+}
+
+// ----------------------------------------------------------------------------------------------
+// qt[b,h,rho] = sum_d q[b,h,d] * B[b,h/G,rho,d]; one workgroup per (kv head, batch), one thread
+// per rho (strided), the G query rows of the kv head held in LDS as fp32.
+// ----------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void absorb_q_kernel(
+    const T* __restrict__ q, const T* __restrict__ B, T* __restrict__ qt_hi, T* __restrict__ qt_lo,
+    int hq, int hkv, int d, int rank, int64_t sBb, int64_t sBh, int64_t sBr) {
+  typedef typename Elem<T>::vec8 vec8;
+  __shared__ float qs[32 * 256];
+  const int kh = blockIdx.x, b = blockIdx.y, G = hq / hkv;
+  const T* qb = q + ((int64_t)b * hq + (int64_t)kh * G) * d;
+  for (int i = threadIdx.x; i < G * d; i += blockDim.x) qs[i] = to_f32(qb[i]);
+  __syncthreads();
+  const T* Bh = B + b * sBb + kh * sBh;
+  for (int rho = threadIdx.x; rho < rank; rho += blockDim.x) {
+    const T* row = Bh + rho * sBr;
+    for (int g0 = 0; g0 < G; g0 += 4) {
+      float acc[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int c = 0; c < d; c += 8) {
+        vec8 v = ld16<vec8>(row + c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float x = to_f32(v[e]);
+#pragma unroll
+          for (int gi = 0; gi < 4; ++gi)
+            if (g0 + gi < G) acc[gi] += x * qs[(g0 + gi) * d + c + e];
+        }
+      }
+#pragma unroll
+      for (int gi = 0; gi < 4; ++gi)
+        if (g0 + gi < G) {
+          int64_t o = ((int64_t)b * hq + (int64_t)kh * G + g0 + gi) * rank + rho;
+          T hi = from_f32<T>(acc[gi]);
+          qt_hi[o] = hi;
+          if (qt_lo) qt_lo[o] = from_f32<T>(acc[gi] - to_f32(hi));
+        }
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------------------------
+// Stage 2.  One workgroup per (kv head, batch): merges the live splits of its G query heads
+// (reference order: increasing split id, running max of lse), then optionally multiplies the
+// merged rank-space rows by vB[b, kh] (read once for the G heads).
+// ----------------------------------------------------------------------------------------------
+template <typename O, typename TB>
+__global__ __launch_bounds__(256) void merge_stage2_kernel(
+    const float* __restrict__ partial, const float* __restrict__ lse, O* __restrict__ out,
+    const TB* __restrict__ vB, int64_t sVb, int64_t sVh, int64_t sVr, int d_out,
+    const int32_t* __restrict__ num_kv_splits, const int32_t* __restrict__ kv_lens,
+    int hq, int hkv, int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh) {
+  extern __shared__ float merged[];  // [G][dv]
+  const int kh = blockIdx.x, b = blockIdx.y, G = hq / hkv;
+  const int L = kv_lens ? kv_lens[b] : kv_len;
+  const int ns = num_kv_splits[b];
+  for (int idx = threadIdx.x; idx < G * dv; idx += blockDim.x) {
+    const int gi = idx / dv, c = idx - gi * dv;
+    const int h = kh * G + gi;
+    const float* pl = lse + ((int64_t)b * hq + h) * max_splits;
+    const float* pp = partial + ((int64_t)b * hq + h) * max_splits * (int64_t)dv + c;
+    float g_lse = NEG_INF, g_sum = 0.f, acc = 0.f;
+    for (int i = 0; i < max_splits; ++i) {
+      int s, e;
+      split_bounds(L, ns, i, s, e);
+      if (e > s) {
+        float tv = pp[(int64_t)i * dv];
+        float in = pl[i];
+        float nl = fmaxf(in, g_lse);
+        float old_scale = __expf(g_lse - nl);
+        float w = __expf(in - nl);
+        acc = acc * old_scale + w * tv;
+        g_sum = g_sum * old_scale + w;
+        g_lse = nl;
+      }
+    }
+    float r = acc / g_sum;
+    if (vB)
+      merged[idx] = r;
+    else
+      out[b * sOb + h * sOh + c] = (O)r;
+  }
+  if (!vB) return;
+  __syncthreads();
+  const TB* Bh = vB + b * sVb + kh * sVh;
+  // thread -> (output column, rank slice); slices reduced through LDS atomics-free tree
+  const int nsl = blockDim.x / d_out;  // d_out <= 256 -> nsl >= 1
+  const int col = threadIdx.x % d_out, sl = threadIdx.x / d_out;
+  __shared__ float red[256 * 16];
+  float acc[16];
+  for (int gi = 0; gi < G; ++gi) acc[gi] = 0.f;
+  if (sl < nsl) {
+    for (int rho = sl; rho < dv; rho += nsl) {
+      float w = to_f32(Bh[rho * sVr + col]);
+      for (int gi = 0; gi < G; ++gi) acc[gi] += merged[gi * dv + rho] * w;
+    }
+  }
+  for (int gi = 0; gi < G; ++gi) red[gi * 256 + threadIdx.x] = (sl < nsl) ? acc[gi] : 0.f;
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < G * d_out; idx += blockDim.x) {
+    const int gi = idx / d_out, c = idx - gi * d_out;
+    float s = 0.f;
+    for (int k = 0; k < nsl; ++k) s += red[gi * 256 + k * d_out + c];
+    out[b * sOb + (kh * G + gi) * sOh + c] = (O)s;
+  }
+}
+
+template <typename O>
+static int launch_rope(void* s, void* c, const float* inv, int64_t seqlen, int64_t start, int half_dim,
+                       hipStream_t st) {
+  int64_t n = seqlen * half_dim;
+  rope_table_kernel<O><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>((O*)s, (O*)c, inv, seqlen, start,
+                                                                               half_dim);
+  return launch_status();
+}
+
+template <typename O, typename TB>
+static int launch_merge(const float* partial, const float* lse, void* out, const void* vB, int64_t sVb, int64_t sVh,
+                        int64_t sVr, int d_out, const int32_t* ns, const int32_t* kl, int batch, int hq, int hkv,
+                        int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, hipStream_t st) {
+  size_t shm = (size_t)(hq / hkv) * dv * sizeof(float);
+  merge_stage2_kernel<O, TB><<<dim3(hkv, batch), dim3(256), shm, st>>>(partial, lse, (O*)out, (const TB*)vB, sVb, sVh,
+                                                                      sVr, d_out, ns, kl, hq, hkv, kv_len, max_splits,
+                                                                      dv, sOb, sOh);
+  return launch_status();
+}
+
+}  // namespace xkv
+
+using namespace xkv;
+
+extern "C" int xkv_abi_version(void) { return XKV_ABI_VERSION; }
+
+extern "C" const char* xkv_error_string(int code) {
+  switch (code) {
+    case XKV_OK: return "ok";
+    case XKV_EINVAL: return "invalid argument (null pointer or non-positive size)";
+    case XKV_EUNSUPPORTED: return "shape outside the built envelope";
+    case XKV_EALIGN: return "pointer or stride not 16-byte aligned";
+    case XKV_EDTYPE: return "unsupported dtype code";
+    default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown xkv error";
+  }
+}
+
+extern "C" int xkv_rope_table(void* sin_out, void* cos_out, const float* inv_freq, int64_t seqlen, int64_t start,
+                              int half_dim, int out_dtype, void* stream) {
+  if (!sin_out || !cos_out || !inv_freq || seqlen < 0 || half_dim <= 0) return XKV_EINVAL;
+  if (seqlen == 0) return XKV_OK;
+  hipStream_t st = (hipStream_t)stream;
+  switch (out_dtype) {
+    case XKV_F32: return launch_rope<float>(sin_out, cos_out, inv_freq, seqlen, start, half_dim, st);
+    case XKV_F16: return launch_rope<_Float16>(sin_out, cos_out, inv_freq, seqlen, start, half_dim, st);
+    case XKV_BF16: return launch_rope<__bf16>(sin_out, cos_out, inv_freq, seqlen, start, half_dim, st);
+    default: return XKV_EDTYPE;
+  }
+}
+
+extern "C" int xkv_absorb_q(const void* q, const void* B, void* qt_hi, void* qt_lo, int batch, int hq, int hkv, int d,
+                            int rank, int64_t sBb, int64_t sBh, int64_t sBr, int dtype, void* stream) {
+  if (!q || !B || !qt_hi || batch <= 0 || hq <= 0 || hkv <= 0 || d <= 0 || rank <= 0) return XKV_EINVAL;
+  if (hq % hkv || hq / hkv > 32 || d > 256 || d % 8) return XKV_EUNSUPPORTED;
+  if (sBr % 8 || sBh % 8 || sBb % 8 || ((uintptr_t)B & 15)) return XKV_EALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid(hkv, batch), block(256);
+  if (dtype == XKV_BF16)
+    absorb_q_kernel<__bf16><<<grid, block, 0, st>>>((const __bf16*)q, (const __bf16*)B, (__bf16*)qt_hi, (__bf16*)qt_lo,
+                                                    hq, hkv, d, rank, sBb, sBh, sBr);
+  else if (dtype == XKV_F16)
+    absorb_q_kernel<_Float16><<<grid, block, 0, st>>>((const _Float16*)q, (const _Float16*)B, (_Float16*)qt_hi,
+                                                      (_Float16*)qt_lo, hq, hkv, d, rank, sBb, sBh, sBr);
+  else
+    return XKV_EDTYPE;
+  return launch_status();
+}
+
+extern "C" int xkv_merge_stage2(const float* partial, const float* lse, void* out, const void* vB, int64_t sVb,
+                                int64_t sVh, int64_t sVr, int d_out, int vB_dtype, const int32_t* ns,
+                                const int32_t* kl, int batch, int hq, int hkv, int kv_len, int max_splits, int dv,
+                                int64_t sOb, int64_t sOh, int out_dtype, void* stream) {
+  if (!partial || !lse || !out || !ns || batch <= 0 || hq <= 0 || hkv <= 0 || max_splits <= 0 || dv <= 0)
+    return XKV_EINVAL;
+  if (hq % hkv || hq / hkv > 16 || dv > 512) return XKV_EUNSUPPORTED;
+  if (vB && (d_out <= 0 || d_out > 256)) return XKV_EUNSUPPORTED;
+  hipStream_t st = (hipStream_t)stream;
+#define XKV_MERGE(O, TB) \
+  return launch_merge<O, TB>(partial, lse, out, vB, sVb, sVh, sVr, d_out, ns, kl, batch, hq, hkv, kv_len, max_splits, dv, sOb, sOh, st)
+  const int bt = vB ? vB_dtype : XKV_BF16;
+  if (bt != XKV_BF16 && bt != XKV_F16) return XKV_EDTYPE;
+  switch (out_dtype) {
+    case XKV_F32: if (bt == XKV_BF16) XKV_MERGE(float, __bf16); else XKV_MERGE(float, _Float16);
+    case XKV_F16: if (bt == XKV_BF16) XKV_MERGE(_Float16, __bf16); else XKV_MERGE(_Float16, _Float16);
+    case XKV_BF16: if (bt == XKV_BF16) XKV_MERGE(__bf16, __bf16); else XKV_MERGE(__bf16, _Float16);
+    default: return XKV_EDTYPE;
+  }
+#undef XKV_MERGE
+}

@@ -1,0 +1,87 @@
+// Shared device helpers for the xKV decode kernels (gfx950 / CDNA4 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/xkv_hip.h"
+
+namespace xkv {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned short u16;
+
+constexpr int WAVE = 64;
+constexpr int MIN_BLOCK_KV = 32;  // split granularity, flash_decoding/gqa.py:38 of the reference
+constexpr float NEG_INF = -__builtin_huge_valf();
+
+// 16-bit operand type traits.  A "packet" is 8 consecutive elements = 16 bytes =
+// one lane's share of a 16x16x32 (or 32x32x16) MFMA operand.
+template <typename T> struct Elem;
+template <> struct Elem<__bf16> {
+  typedef bf16x8 vec8;
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Elem<_Float16> {
+  typedef f16x8 vec8;
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
+template <typename T> __device__ __forceinline__ T from_f32(float x) { return (T)x; }
+
+__device__ __forceinline__ u16 bits_of(__bf16 x) { return __builtin_bit_cast(u16, x); }
+__device__ __forceinline__ u16 bits_of(_Float16 x) { return __builtin_bit_cast(u16, x); }
+
+// 16-byte packet load/store through a generic pointer (global or LDS)
+template <typename V> __device__ __forceinline__ V ld16(const void* p) {
+  return __builtin_bit_cast(V, *reinterpret_cast<const u32x4*>(p));
+}
+template <typename V> __device__ __forceinline__ void st16(void* p, V v) {
+  *reinterpret_cast<u32x4*>(p) = __builtin_bit_cast(u32x4, v);
+}
+
+__host__ __device__ __forceinline__ int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// Token range of one KV split; identical integer arithmetic to the reference's
+// flash_decoding/gqa.py:95-99 (stage 1) and :273-281 (stage 2).
+__host__ __device__ __forceinline__ void split_bounds(int kv_len, int num_splits, int split_id,
+                                                       int& start, int& end) {
+  int per = cdiv(cdiv(kv_len, num_splits), MIN_BLOCK_KV) * MIN_BLOCK_KV;
+  start = per * split_id;
+  int e = start + per;
+  end = e < kv_len ? e : kv_len;
+}
+
+// Reductions over the 4 lane groups {n, n+16, n+32, n+48} that share a column
+// index in the 16x16 MFMA result layout.
+__device__ __forceinline__ float group4_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16));
+  v = fmaxf(v, __shfl_xor(v, 32));
+  return v;
+}
+__device__ __forceinline__ float group4_sum(float v) {
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  return v;
+}
+
+inline int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? XKV_OK : (int)e;
+}
+
+}  // namespace xkv

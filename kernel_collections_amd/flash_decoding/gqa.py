@@ -1,0 +1,65 @@
+"""Split-K flash decoding for grouped-query attention on plain K/V buffers.
+
+Call surface of the reference's flash_decoding/gqa.py:339-434 (``decode_attention_fwd``), plus
+  * ``kv_lens``: optional int32 ``[batch]`` of per-sequence lengths (ragged batch; the reference has
+    one length, ``k_buffer.shape[1]``, for the whole batch - gqa.py:60,194);
+  * ``decode_attention_fwd_v_factorized``: K plain, ``V = v_A @ v_B`` (the eager semantics of
+    ``group_query_attention_factorized_v_only``, reference attention.py:202-274) as a split-K kernel
+    that accumulates ``P @ v_A`` in rank space and multiplies by ``v_B`` after the merge.
+Split ranges follow gqa.py:95-99 exactly; ``sm_scale`` multiplies the scores (gqa.py:122).
+"""
+from __future__ import annotations
+
+from kernel_collections_amd import ops
+
+
+def _prep(q, k_buffer, num_kv_splits, max_kv_splits, kv_lens):
+    assert q.dim() == 3 and k_buffer.dim() == 4
+    batch, num_q_heads, head_dim = q.shape
+    num_kv_heads = k_buffer.shape[2]
+    assert k_buffer.shape[0] == batch and k_buffer.shape[-1] == head_dim
+    kv_group_num = num_q_heads // num_kv_heads
+    assert kv_group_num >= 1 and num_q_heads % num_kv_heads == 0
+    assert kv_group_num <= 32, "at most 32 query heads per kv head"
+    assert head_dim % 32 == 0, "head_dim must be a multiple of 32"
+    splits = ops.as_int32_dev(num_kv_splits, batch, q.device)
+    lens = None if kv_lens is None else ops.as_int32_dev(kv_lens, batch, q.device)
+    return batch, num_q_heads, num_kv_heads, head_dim, int(max_kv_splits), splits, lens
+
+
+def decode_attention_fwd(q, k_buffer, v_buffer, o, num_kv_splits, max_kv_splits, sm_scale=1.0, *, kv_lens=None):
+    """q ``[batch, Hq, d]``; k_buffer / v_buffer ``[batch, kv_len, Hkv, d]``; o ``[batch, Hq, d]`` (filled,
+    returned); num_kv_splits int32 ``[batch]`` on the device; max_kv_splits int."""
+    batch, hq, hkv, d, S, splits, lens = _prep(q, k_buffer, num_kv_splits, max_kv_splits, kv_lens)
+    ops.check_16bit(q, k_buffer, v_buffer)
+    assert k_buffer.shape[-1] == v_buffer.shape[-1], "head dim of K and V must be the same"
+    dv = v_buffer.shape[-1]
+    assert dv % 64 == 0 and dv <= 512
+    kv_len = k_buffer.shape[1]
+    q3 = ops._q3(q)
+    k_buffer, v_buffer = ops.as_rows(k_buffer), ops.as_rows(v_buffer)
+    partial, lse = ops.workspaces(batch, hq, S, dv, q.device)
+    ops.latent_stage1(q3, None, None,
+                      (k_buffer, k_buffer.stride(0), k_buffer.stride(1), k_buffer.stride(2), d), None,
+                      (v_buffer, v_buffer.stride(0), v_buffer.stride(1), v_buffer.stride(2), dv),
+                      partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale))
+    return ops.merge_stage2(partial, lse, o, None, splits, lens, batch, hq, hq, kv_len, S)
+
+
+def decode_attention_fwd_v_factorized(q, k_buffer, v_A_buffer, v_B_buffer, o, num_kv_splits, max_kv_splits,
+                                      sm_scale=1.0, *, kv_lens=None):
+    """K plain ``[batch, kv_len, Hkv, d]``; v_A ``[batch, kv_len, rv]``; v_B ``[batch, Hkv, rv, d]``."""
+    batch, hq, hkv, d, S, splits, lens = _prep(q, k_buffer, num_kv_splits, max_kv_splits, kv_lens)
+    ops.check_16bit(q, k_buffer, v_A_buffer, v_B_buffer)
+    rv = v_A_buffer.shape[-1]
+    assert v_A_buffer.shape[1] == k_buffer.shape[1] and v_B_buffer.shape[1] == hkv and v_B_buffer.shape[2] == rv
+    assert rv % 64 == 0 and rv <= 512
+    kv_len = k_buffer.shape[1]
+    q3 = ops._q3(q)
+    k_buffer, v_A_buffer = ops.as_rows(k_buffer), ops.as_rows(v_A_buffer)
+    partial, lse = ops.workspaces(batch, hq, S, rv, q.device)
+    ops.latent_stage1(q3, None, None,
+                      (k_buffer, k_buffer.stride(0), k_buffer.stride(1), k_buffer.stride(2), d), None,
+                      (v_A_buffer, v_A_buffer.stride(0), v_A_buffer.stride(1), 0, rv),
+                      partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale))
+    return ops.merge_stage2(partial, lse, o, v_B_buffer, splits, lens, batch, hq, hkv, kv_len, S)

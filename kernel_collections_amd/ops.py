@@ -1,0 +1,176 @@
+"""Thin host layer over the C ABI: marshals torch tensors into the `xkv_*` entry points.
+
+Everything here launches HIP kernels on the current stream and returns without synchronising.
+Workspaces are `torch.empty` tensors owned by the caller's allocator; the C side allocates nothing.
+"""
+from __future__ import annotations
+
+from ctypes import c_float, c_int, c_int64, c_void_p
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import check, dtype_code, kv_operand, ptr, q_operand, stream_ptr
+
+_16BIT = (torch.float16, torch.bfloat16)
+_NUM_CU = 256  # MI355X
+
+
+def _cdiv(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+# ------------------------------------------------------------------------------------------------
+# small cached device constants (no per-call host->device traffic on the hot path)
+# ------------------------------------------------------------------------------------------------
+_inv_freq_cache = {}
+_splits_cache = {}
+
+
+def rope_inv_freq(dim: int, theta: float, device) -> torch.Tensor:
+    """fp32 `theta**(-2j/dim)` evaluated exactly as the reference's eager RoPE does on the host
+    (flash_recontruction/rope/rope_ref.py:4), cached per (dim, theta, device)."""
+    key = (int(dim), float(theta), str(device))
+    t = _inv_freq_cache.get(key)
+    if t is None:
+        inv = 1.0 / (float(theta) ** (torch.arange(0, dim, 2, dtype=torch.int64).float() / dim))
+        t = inv.to(device=device, dtype=torch.float32).contiguous()
+        _inv_freq_cache[key] = t
+    return t
+
+
+def uniform_splits(batch: int, n: int, device) -> torch.Tensor:
+    """int32 `[batch]` tensor filled with `n` (what the reference builds with torch.ones(...)*128,
+    flash_decoding/mla2/mla_flash_decoding.py:20), cached."""
+    key = (int(batch), int(n), str(device))
+    t = _splits_cache.get(key)
+    if t is None:
+        t = torch.full((batch,), int(n), dtype=torch.int32, device=device)
+        _splits_cache[key] = t
+    return t
+
+
+def occupancy_splits(batch: int, groups: int, kv_len: int, tile: int = 64, waves: int = 2) -> int:
+    """Number of KV splits that gives about `waves` workgroups per CU without making a split
+    shorter than 4 tiles."""
+    want = _cdiv(waves * _NUM_CU, max(1, batch * groups))
+    cap = max(1, kv_len // (4 * tile))
+    return max(1, min(want, cap))
+
+
+def _row_ok(t: torch.Tensor) -> bool:
+    """Unit stride on the feature axis, every other stride a multiple of 8 elements, 16-byte base."""
+    if t.stride(-1) != 1 or t.data_ptr() % 16:
+        return False
+    return all(s % 8 == 0 for s in t.stride()[:-1])
+
+
+def as_rows(t: torch.Tensor) -> torch.Tensor:
+    return t if _row_ok(t) else t.contiguous()
+
+
+def _q3(q: torch.Tensor) -> torch.Tensor:
+    q = q.contiguous()
+    assert q.data_ptr() % 16 == 0
+    return q
+
+
+# ------------------------------------------------------------------------------------------------
+# entry-point wrappers
+# ------------------------------------------------------------------------------------------------
+def rope_table(seqlen: int, theta: float, start: int, dtype, device, half_dim: int = 64):
+    sin = torch.empty((seqlen, half_dim), dtype=dtype, device=device)
+    cos = torch.empty_like(sin)
+    inv = rope_inv_freq(2 * half_dim, theta, sin.device)
+    check(_lib.lib().xkv_rope_table(ptr(sin), ptr(cos), ptr(inv), c_int64(seqlen), c_int64(start), half_dim,
+                                    dtype_code(dtype), stream_ptr(sin)), "xkv_rope_table")
+    return sin, cos
+
+
+def absorb_q(q3: torch.Tensor, Bk: torch.Tensor, want_lo: bool = True) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """q3 `[b,Hq,d]`, Bk `[b,Hkv,r,d]` (any batch/head/rank strides) -> q~ hi (and lo) `[b,Hq,r]`."""
+    b, hq, d = q3.shape
+    _, hkv, r, _ = Bk.shape
+    Bk = as_rows(Bk)
+    hi = torch.empty((b, hq, r), dtype=q3.dtype, device=q3.device)
+    lo = torch.empty_like(hi) if want_lo else None
+    check(_lib.lib().xkv_absorb_q(ptr(q3), ptr(Bk), ptr(hi), ptr(lo), b, hq, hkv, d, r,
+                                  c_int64(Bk.stride(0)), c_int64(Bk.stride(1)), c_int64(Bk.stride(2)),
+                                  dtype_code(q3.dtype), stream_ptr(q3)), "xkv_absorb_q")
+    return hi, lo
+
+
+def latent_stage1(qn, qn_lo, qr, C, R, V, partial, lse, scores, num_kv_splits, kv_lens,
+                  batch, hq, groups, kv_len, max_splits, sm_scale, logit_cap=0.0):
+    """C / R / V are `(tensor, stride_b, stride_l, stride_h, dim)` tuples or None."""
+    def op(x):
+        return kv_operand(None) if x is None else kv_operand(*x)
+    sd = dtype_code(scores.dtype) if scores is not None else 0
+    check(_lib.lib().xkv_latent_stage1(
+        q_operand(qn), ptr(qn_lo), q_operand(qr), op(C), op(R), op(V), ptr(partial), ptr(lse), ptr(scores), sd,
+        ptr(num_kv_splits), ptr(kv_lens), batch, hq, groups, kv_len, max_splits,
+        c_float(sm_scale), c_float(logit_cap), dtype_code(qn.dtype), stream_ptr(qn)), "xkv_latent_stage1")
+
+
+def recon_stage1(q3, kA, kB, vA, partial, lse, scores, num_kv_splits, kv_lens, batch, hq, hkv, kv_len, max_splits,
+                 sm_scale, rope, inv_freq, pos_offset, sin_cos):
+    a_op = kv_operand(kA, kA.stride(0), kA.stride(1), 0, kA.shape[-1])
+    v_op = kv_operand(None) if vA is None else kv_operand(vA, vA.stride(0), vA.stride(1), 0, vA.shape[-1])
+    sd = dtype_code(scores.dtype) if scores is not None else 0
+    check(_lib.lib().xkv_recon_stage1(
+        ptr(q3), a_op, ptr(kB), c_int64(kB.stride(0)), c_int64(kB.stride(1)), c_int64(kB.stride(2)), v_op,
+        ptr(partial), ptr(lse), ptr(scores), sd, ptr(num_kv_splits), ptr(kv_lens), batch, hq, hkv, kv_len, max_splits,
+        c_float(sm_scale), int(rope), ptr(inv_freq), c_int64(pos_offset), ptr(sin_cos),
+        c_int64(sin_cos.stride(0) if sin_cos is not None else 0), dtype_code(q3.dtype), stream_ptr(q3)),
+        "xkv_recon_stage1")
+
+
+def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, kv_len, max_splits):
+    """out `[b,Hq,*]` (strides honoured on the first two axes)."""
+    dv = partial.shape[-1]
+    assert out.stride(-1) == 1
+    if vB is not None:
+        vB = as_rows(vB)
+        sv = (vB.stride(0), vB.stride(1), vB.stride(2))
+        d_out, vdt = vB.shape[-1], dtype_code(vB.dtype)
+    else:
+        sv, d_out, vdt = (0, 0, 0), dv, _lib.XKV_BF16
+    check(_lib.lib().xkv_merge_stage2(
+        ptr(partial), ptr(lse), ptr(out), ptr(vB), c_int64(sv[0]), c_int64(sv[1]), c_int64(sv[2]), d_out, vdt,
+        ptr(num_kv_splits), ptr(kv_lens), batch, hq, hkv, kv_len, max_splits, dv,
+        c_int64(out.stride(0)), c_int64(out.stride(1)), dtype_code(out.dtype), stream_ptr(partial)),
+        "xkv_merge_stage2")
+    return out
+
+
+def workspaces(batch: int, hq: int, max_splits: int, dv: int, device):
+    partial = torch.empty((batch, hq, max_splits, dv), dtype=torch.float32, device=device)
+    lse = torch.empty((batch, hq, max_splits), dtype=torch.float32, device=device)
+    return partial, lse
+
+
+def head_groups(hq: int, limit: int = 32) -> int:
+    """Smallest number of equal head groups with at most `limit` heads each."""
+    g = _cdiv(hq, limit)
+    while hq % g:
+        g += 1
+    return g
+
+
+def check_16bit(*ts):
+    dt = ts[0].dtype
+    assert dt in _16BIT, f"xkv HIP kernels take float16 or bfloat16 operands, got {dt}"
+    for t in ts:
+        if t is not None:
+            assert t.dtype == dt, f"operand dtypes differ: {t.dtype} vs {dt}"
+            _lib.require_gpu(t)
+
+
+def as_int32_dev(x, batch: int, device) -> torch.Tensor:
+    if torch.is_tensor(x):
+        assert x.numel() == batch
+        if x.dtype != torch.int32 or x.device != device:
+            x = x.to(device=device, dtype=torch.int32)
+        return x.contiguous()
+    return uniform_splits(batch, int(x), device)

@@ -1,0 +1,119 @@
+"""CPU-side checks of the drop-in boundary: the C-ABI library loads and exports exactly the symbols
+include/xkv_hip.h declares (no compute call is made), argument validation answers before any launch,
+and the Python mirrors expose the reference's names and signatures."""
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "xkv_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(xkv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from kernel_collections_amd import _lib
+    names = _declared()
+    assert set(names) == set(_lib.EXPORTS), (names, _lib.EXPORTS)
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} not exported"
+    assert _lib.lib().xkv_abi_version() == _lib.ABI_VERSION
+    assert _lib.lib().xkv_error_string(0) == b"ok"
+    assert b"envelope" in _lib.lib().xkv_error_string(-2)
+
+
+def test_argument_errors_are_reported_before_any_launch():
+    from kernel_collections_amd import _lib
+    L = _lib.lib()
+    null = ctypes.c_void_p(0)
+    assert L.xkv_rope_table(null, null, null, 4, 0, 64, _lib.XKV_F32, null) == -1
+    assert L.xkv_absorb_q(null, null, null, null, 1, 4, 2, 128, 64, 0, 0, 0, _lib.XKV_BF16, null) == -1
+    q = _lib.QOperand(ctypes.c_void_p(16), 100)
+    kv = _lib.KVOperand(ctypes.c_void_p(16), 0, 100, 0, 100)
+    none = _lib.KVOperand(null, 0, 0, 0, 0)
+    ns = ctypes.c_void_p(16)
+    # feature width 100 is outside the envelope (multiple of 32 required)
+    rc = L.xkv_latent_stage1(q, null, _lib.QOperand(null, 0), kv, none, kv, ctypes.c_void_p(16), ctypes.c_void_p(16),
+                             null, 0, ns, null, 1, 4, 1, 8, 1, 1.0, 0.0, _lib.XKV_BF16, null)
+    assert rc == -2
+    with pytest.raises(RuntimeError, match="envelope"):
+        _lib.check(rc, "xkv_latent_stage1")
+
+
+def test_python_surface_matches_reference_names_and_argument_order():
+    import kernel_collections_amd.flash_recontruction as fr
+    from kernel_collections_amd.flash_decoding import gqa, mla, mla2
+    for n in ("qAB_no_pe_v1", "qAB_no_pe_v2", "qAB_no_pe_ref", "qAB_rope_v1", "qAB_rope_v2", "qAB_rope_v3",
+              "qAB_rope_v4", "gqa_xKV_no_pe_ref", "gqa_xKV_no_pe_k_only_ref", "gqa_xKV_no_pe_k_only",
+              "gqa_xKV_no_pe", "gqa_xKV_no_pe_v2"):
+        assert n in fr.__all__ and callable(getattr(fr, n))
+    pos = lambda f: [p.name for p in inspect.signature(f).parameters.values()
+                     if p.kind == p.POSITIONAL_OR_KEYWORD]
+    assert pos(fr.qAB_no_pe_v1) == ["q", "Ak", "Bk"]
+    assert pos(fr.qAB_rope_v1) == ["q", "Ak", "Bk", "theta"]
+    assert inspect.signature(fr.qAB_rope_v1).parameters["theta"].default == 10000000.0
+    assert pos(fr.qAB_rope_v2) == ["q", "Ak", "Bk", "sin_cos"]
+    assert pos(fr.gqa_xKV_no_pe) == ["q", "k_A_buffer", "k_B_buffer", "v_A_buffer", "v_B_buffer", "o",
+                                     "num_kv_splits", "max_kv_splits", "sm_scale"]
+    assert pos(fr.gqa_xKV_no_pe_v2) == ["q", "k_A_buffer", "k_B_buffer", "v_A_buffer", "v_B_buffer",
+                                        "num_kv_splits", "max_kv_splits", "sm_scale"]
+    assert pos(fr.gqa_xKV_no_pe_k_only) == ["q", "k_A_buffer", "k_B_buffer", "v_buffer", "o", "num_kv_splits",
+                                            "max_kv_splits", "sm_scale"]
+    assert pos(gqa.decode_attention_fwd) == ["q", "k_buffer", "v_buffer", "o", "num_kv_splits", "max_kv_splits",
+                                             "sm_scale"]
+    assert pos(mla.decode_attention_fwd) == ["q", "k_buffer", "v_buffer", "o", "sm_scale", "logit_cap"]
+    assert pos(mla2.mla_decode_attention_fwd) == ["q_nope", "q_rope", "kv_nope", "k_rope", "sm_scale"]
+    assert pos(mla2.mla_decode_attention_xKV) == ["q_nope", "q_rope", "kv_A_nope", "kv_B_nope", "k_rope", "sm_scale"]
+    from kernel_collections_amd.flash_recontruction.rope.sin_cos import rotary_sin_cos
+    assert pos(rotary_sin_cos) == ["seqlen", "theta", "starting_idx"]
+
+
+def test_reference_asserts_are_kept():
+    import kernel_collections_amd.flash_recontruction as fr
+    q = torch.zeros(1, 4, 2, 128, dtype=torch.bfloat16)
+    A = torch.zeros(1, 8, 64, dtype=torch.bfloat16)
+    B = torch.zeros(1, 2, 64, 128, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="q_len=1"):
+        fr.qAB_no_pe_v1(q, A, B)
+    with pytest.raises(AssertionError, match="Rank mismatch"):
+        fr.qAB_rope_v1(q[:, :, :1], A, torch.zeros(1, 2, 32, 128, dtype=torch.bfloat16))
+    with pytest.raises(AssertionError, match="4D"):
+        fr.qAB_no_pe_v1(q[0], A, B)
+    # CPU tensors are refused, never silently computed elsewhere
+    with pytest.raises(AssertionError, match="no CPU path"):
+        fr.qAB_no_pe_v1(q[:, :, :1], A, B)
+
+
+def test_eager_surface_functions_agree_with_the_oracle():
+    import oracle
+    import kernel_collections_amd.flash_recontruction as fr
+    from kernel_collections_amd.flash_decoding import mla, mla2
+    from kernel_collections_amd.flash_recontruction.rope import rope_ref
+    g = torch.Generator().manual_seed(1)
+    r = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    q, A, B, vA, vB = r(2, 8, 1, 16), r(2, 30, 6), r(2, 2, 6, 16), r(2, 30, 10), r(2, 2, 10, 16)
+    assert torch.allclose(fr.qAB_no_pe_ref(q, A, B), oracle.qab_nope(q, A, B))
+    assert torch.allclose(fr.gqa_xKV_no_pe_ref(q[:, :, 0], A, B, vA, vB).float(),
+                          oracle.gqa_xkv(q[:, :, 0], A, B, vA, vB).float(), atol=1e-5)
+    V = r(2, 30, 2, 16)
+    assert torch.allclose(fr.gqa_xKV_no_pe_k_only_ref(q[:, :, 0], A, B, V).float(),
+                          oracle.gqa_xkv_k_only(q[:, :, 0], A, B, V).float(), atol=1e-5)
+    K = r(2, 30, 2, 16)
+    assert torch.allclose(mla.decode_attention_reference(q[:, :, 0], K, V, None, 0.4).float(),
+                          oracle.gqa_plain(q[:, :, 0], K, V, 0.4).float(), atol=1e-5)
+    qn, qr, c, pe = r(2, 4, 12), r(2, 4, 4), r(2, 30, 1, 12), r(2, 30, 1, 4)
+    assert torch.allclose(mla2.mla_decode_attention_fwd_ref(qn, qr, c, pe, 0.3).float(),
+                          oracle.mla_ref(qn, qr, c, pe, 0.3).float(), atol=1e-5)
+    cos, sin = rope_ref.LlamaRotaryEmbedding(128, 50, 5e5)
+    ocos, osin = oracle.rope_cos_sin(torch.arange(50), 128, 5e5)
+    assert torch.equal(cos, ocos) and torch.equal(sin, osin)
+    x = r(50, 128).float()
+    assert torch.equal(rope_ref.apply_rotary_pos_emb_pytorch(x, cos, sin)[0], oracle.apply_rope(x, ocos, osin))
