@@ -115,6 +115,9 @@ int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_operand qr,
  * then either scores_out (as above) or the split softmax with V = vA (rank-space partials
  * [batch, hq, max_splits, vA.dim]).  rope == 0 skips the rotation (pure reconstruction).
  * Envelope: head_dim == 128, G = hq/hkv <= 16, rank % 32 == 0, rank <= 512, vA.dim % 64 == 0 <= 512.
+ * With rank == 512, vA the same tensor as kA, computed angles (sin_cos == NULL), G <= 8 and a workspace of
+ * xkv_recon_workspace_bytes() the call runs the specialised kernel (kB packed once into the workspace, 2 x 2
+ * rank/feature wave split on v_mfma_f32_32x32x16, async direct-to-LDS tile ring); otherwise the generic one.
  * Replaces _qAB_fwd[grid] at flash_recontruction/qAB/v1.py:135-145 (v3.py / v4.py / ref.py twins) and
  * _qAB_fwd_precomp[grid] at qAB/v2.py:170-186 in scores_out mode; the fused form has no single
  * reference launch - it composes that reconstruction with the stage 1 of
@@ -128,7 +131,13 @@ int xkv_recon_stage1(const void* q_pe, xkv_kv_operand kA, const void* kB,
                      int batch, int hq, int hkv, int kv_len, int max_splits,
                      float sm_scale, int rope, const float* inv_freq, int64_t pos_offset,
                      const void* sin_cos, int64_t sc_stride_l,
+                     void* workspace, int64_t workspace_bytes,
                      int dtype, void* stream);
+
+/* Bytes of caller-owned scratch that lets xkv_recon_stage1 take its MFMA-bound fast path (kB re-packed into MFMA
+ * operand order: one copy per batch entry, a single copy when stride_kB_b == 0).  0: no fast path for this rank.
+ * Passing workspace == NULL (or too few bytes) is valid and selects the generic kernel.  No reference counterpart. */
+int64_t xkv_recon_workspace_bytes(int batch, int hkv, int rank, int64_t stride_kB_b);
 
 /* Stage 2: LSE-weighted merge of the live splits in increasing split id,
  *   out[b,h,:] = sum_i w_i partial[b,h,i,:] / sum_i w_i ,  w_i = exp(lse_i - max lse),

@@ -16,7 +16,7 @@ ABI_VERSION = 1
 
 EXPORTS = (
     "xkv_abi_version", "xkv_error_string", "xkv_rope_table", "xkv_absorb_q",
-    "xkv_latent_stage1", "xkv_recon_stage1", "xkv_merge_stage2",
+    "xkv_latent_stage1", "xkv_recon_stage1", "xkv_recon_workspace_bytes", "xkv_merge_stage2",
 )
 
 
@@ -50,7 +50,9 @@ def _declare(lib):
     lib.xkv_recon_stage1.argtypes = [c_void_p, KVOperand, c_void_p, c_int64, c_int64, c_int64, KVOperand,
                                      c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_int64,
-                                     c_void_p, c_int64, c_int, c_void_p]
+                                     c_void_p, c_int64, c_void_p, c_int64, c_int, c_void_p]
+    lib.xkv_recon_workspace_bytes.restype = c_int64
+    lib.xkv_recon_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int64]
     lib.xkv_merge_stage2.restype = c_int
     lib.xkv_merge_stage2.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,

@@ -1,0 +1,21 @@
+// Interface between the recon stage-1 dispatcher and its MFMA-bound fast path (recon_fast.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace xkv {
+
+struct FastParams {
+  const void* q; const void* kA; const void* Bp;   // Bp: kB re-packed into MFMA operand order (caller workspace)
+  int64_t sAb, sAl, sBpb;
+  float* partial; float* lse;
+  const int32_t* num_splits; const int32_t* kv_lens;
+  int hq, hkv, kv_len, max_splits, total_wg;
+  float sm_scale;
+  const float* inv_freq; int64_t pos_offset;
+};
+
+int launch_recon_fast(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
+                      hipStream_t st);
+
+}  // namespace xkv

@@ -17,6 +17,7 @@
 // in-tile offset (0..31) times a per-tile base rotation that is re-seeded with a fully
 // range-reduced sincosf every 32 tiles and advanced by a constant rotation in between.
 #include "xkv_common.h"
+#include "recon_fast.h"
 
 namespace xkv {
 
@@ -358,12 +359,17 @@ static int dispatch_recon(const ReconParams& p, int batch, bool vshared, hipStre
 
 using namespace xkv;
 
+extern "C" int64_t xkv_recon_workspace_bytes(int batch, int hkv, int rank, int64_t stride_kB_b) {
+  if (rank != 512) return 0;
+  return (int64_t)(stride_kB_b == 0 ? 1 : batch) * hkv * rank * 128 * 2;
+}
+
 extern "C" int xkv_recon_stage1(const void* q_pe, xkv_kv_operand kA, const void* kB, int64_t sBb, int64_t sBh,
                                 int64_t sBr, xkv_kv_operand vA, float* partial, float* lse, void* scores_out,
                                 int scores_dtype, const int32_t* num_kv_splits, const int32_t* kv_lens, int batch,
                                 int hq, int hkv, int kv_len, int max_splits, float sm_scale, int rope,
                                 const float* inv_freq, int64_t pos_offset, const void* sin_cos, int64_t sc_stride_l,
-                                int dtype, void* stream) {
+                                void* workspace, int64_t workspace_bytes, int dtype, void* stream) {
   if (!q_pe || !kA.ptr || !kB || !num_kv_splits || batch <= 0 || hq <= 0 || hkv <= 0 || kv_len <= 0 || max_splits <= 0)
     return XKV_EINVAL;
   const bool so = scores_out != nullptr;
@@ -391,5 +397,17 @@ extern "C" int xkv_recon_stage1(const void* q_pe, xkv_kv_operand kA, const void*
   const bool vshared = !so && vA.ptr == kA.ptr && vA.stride_b == kA.stride_b && vA.stride_l == kA.stride_l &&
                        vA.dim == kA.dim;
   hipStream_t st = (hipStream_t)stream;
+  // MFMA-bound fast path: rank 512, basis shared by K and V, computed RoPE angles, at most 8 query heads per kv head
+  const int64_t need = xkv_recon_workspace_bytes(batch, hkv, rank, sBb);
+  if (!so && vshared && rope && !sin_cos && rank == 512 && hq / hkv <= 8 && workspace && need > 0 &&
+      workspace_bytes >= need && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
+    FastParams f;
+    f.q = q_pe; f.kA = kA.ptr; f.Bp = workspace;
+    f.sAb = kA.stride_b; f.sAl = kA.stride_l; f.sBpb = sBb == 0 ? 0 : (int64_t)hkv * 512 * 128;
+    f.partial = partial; f.lse = lse; f.num_splits = num_kv_splits; f.kv_lens = kv_lens;
+    f.hq = hq; f.hkv = hkv; f.kv_len = kv_len; f.max_splits = max_splits; f.total_wg = batch * hkv * max_splits;
+    f.sm_scale = sm_scale; f.inv_freq = inv_freq; f.pos_offset = pos_offset;
+    return launch_recon_fast(f, kB, sBb, sBh, sBr, batch, dtype, st);
+  }
   return dtype == XKV_BF16 ? dispatch_recon<__bf16>(p, batch, vshared, st) : dispatch_recon<_Float16>(p, batch, vshared, st);
 }

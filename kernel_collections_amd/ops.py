@@ -15,6 +15,7 @@ from ._lib import check, dtype_code, kv_operand, ptr, q_operand, stream_ptr
 
 _16BIT = (torch.float16, torch.bfloat16)
 _NUM_CU = 256  # MI355X
+USE_RECON_WORKSPACE = True  # False: never hand xkv_recon_stage1 a workspace (it then takes its generic kernel)
 
 
 def _cdiv(a: int, b: int) -> int:
@@ -116,13 +117,19 @@ def latent_stage1(qn, qn_lo, qr, C, R, V, partial, lse, scores, num_kv_splits, k
 def recon_stage1(q3, kA, kB, vA, partial, lse, scores, num_kv_splits, kv_lens, batch, hq, hkv, kv_len, max_splits,
                  sm_scale, rope, inv_freq, pos_offset, sin_cos):
     a_op = kv_operand(kA, kA.stride(0), kA.stride(1), 0, kA.shape[-1])
+    ws, ws_bytes = None, 0
+    if scores is None and USE_RECON_WORKSPACE:
+        ws_bytes = _lib.lib().xkv_recon_workspace_bytes(batch, hkv, kA.shape[-1], c_int64(kB.stride(0)))
+        if ws_bytes:
+            ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=q3.device)
     v_op = kv_operand(None) if vA is None else kv_operand(vA, vA.stride(0), vA.stride(1), 0, vA.shape[-1])
     sd = dtype_code(scores.dtype) if scores is not None else 0
     check(_lib.lib().xkv_recon_stage1(
         ptr(q3), a_op, ptr(kB), c_int64(kB.stride(0)), c_int64(kB.stride(1)), c_int64(kB.stride(2)), v_op,
         ptr(partial), ptr(lse), ptr(scores), sd, ptr(num_kv_splits), ptr(kv_lens), batch, hq, hkv, kv_len, max_splits,
         c_float(sm_scale), int(rope), ptr(inv_freq), c_int64(pos_offset), ptr(sin_cos),
-        c_int64(sin_cos.stride(0) if sin_cos is not None else 0), dtype_code(q3.dtype), stream_ptr(q3)),
+        c_int64(sin_cos.stride(0) if sin_cos is not None else 0), ptr(ws), c_int64(ws_bytes),
+        dtype_code(q3.dtype), stream_ptr(q3)),
         "xkv_recon_stage1")
 
 

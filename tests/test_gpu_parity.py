@@ -352,7 +352,8 @@ def test_full_size_config3_properties(dev):
     check_out(o[0], ref0, "config 3, sequence 0")
     perm = torch.arange(b - 1, -1, -1, device=dev)
     o_p = torch.empty_like(o)
-    fr.gqa_xKV_rope(qd[perm], Ad[perm].contiguous(), kBd, Ad[perm].contiguous(), vBd, o_p, ns, S, d ** -0.5, theta)
+    Ap = Ad[perm].contiguous()   # passed as k_A and v_A: one tensor, so the shared-basis kernel runs as above
+    fr.gqa_xKV_rope(qd[perm], Ap, kBd, Ap, vBd, o_p, ns, S, d ** -0.5, theta)
     assert torch.equal(o_p, o[perm]), "sequences are independent: permuting the batch permutes the output bit for bit"
     o2 = torch.empty_like(o)
     fr.gqa_xKV_rope(qd, Ad, kBd, Ad, (vBd * 2).contiguous(), o2, ns, S, d ** -0.5, theta)
