@@ -9,7 +9,7 @@ from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int6
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libxkv_hip.so")
+LIB_PATH = os.environ.get("XKV_HIP_LIB", os.path.join(_HERE, "libxkv_hip.so"))  # override: another build of the same ABI
 
 XKV_F16, XKV_BF16, XKV_F32 = 0, 1, 2
 ABI_VERSION = 1
