@@ -3,9 +3,9 @@
 //
 // Work split.  One workgroup = one (batch, kv head, split); its 4 wavefronts form a 2 x 2 grid over
 // (rank half kq, feature half dq): wave (kq, dq) keeps B[kh][256 kq .. +256][{32 dq .. +32} u {64 + 32 dq .. +32}]
-// stationary in 128 VGPRs (both members of every rotate-half pair) and multiplies it, on
+// stationary in 128 accumulation registers (both members of every rotate-half pair) and multiplies it, on
 // v_mfma_f32_32x32x16, with its rank half of the 32-token tile.  Every element of the tile is therefore read
-// from LDS by two waves, not four - LDS read bandwidth (128 B/clk/CU), not MFMA, bounds the 4-way split.
+// from LDS by two waves, not four - LDS read bandwidth (128 B/clk/CU), not MFMA, bounds a 4-way feature split.
 // RoPE, the rounding to the operand type and the q-dot are all linear in K, so each wave rotates and dots its
 // PARTIAL key tile (partial over its rank half and its feature half) and only 4 x [G x 32] fp32 partial scores
 // are summed through LDS.
@@ -15,17 +15,24 @@
 // (one thread per pair index, incremental rotation re-seeded with a range-reduced sincosf every 32 tiles)
 // and read back as the B operand of the q-dot MFMA.
 //
-// Pipeline.  The tile ring (4 x 32 tokens x 1040 B) is filled by direct-to-LDS loads issued two tiles ahead.
-// Softmax and P.A of tile t-1 run in the same barrier interval as the reconstruction of tile t, so there is ONE
-// workgroup barrier per tile.  The direct-to-LDS loads are inline asm so that the compiler's wait-count pass does
-// not serialise them against every LDS read; completion is tracked by hand (s_waitcnt vmcnt(8): the 8 loads of
-// the next tile may still be in flight).
+// Pipeline.  A wave issues instructions in order, so MFMA time and VALU time only overlap when independent
+// work is interleaved in its instruction stream.  Iteration i therefore runs the reconstruction MFMAs of tile i
+// (accumulating into one of two key-accumulator sets) in three parts, interleaved with what tile i-1 still
+// needs: part 1 rotates tile i-1's partial keys (the other accumulator set) and dots them with q^; part 2 runs
+// the softmax of tile i-1 (wave w owns head w and w+4: no redundant work) and publishes P and the rescale
+// factor through LDS; part 3 accumulates P.A for tile i-1, each wave owning 128 latent features, the token-
+// major operand coming from ds_read_b64_tr_b16.  Three balanced barriers per tile separate the parts.
+// The softmax reference only moves when a tile maximum exceeds it by 16 (lazy rescaling), so the P.A
+// accumulators are almost never rescaled.
+//
+// Tiles stream through a 4-slot LDS ring filled by direct-to-LDS loads issued two tiles ahead.  Those loads
+// are inline asm so that the compiler's wait-count pass does not serialise them against every LDS read;
+// completion is tracked by hand (s_waitcnt vmcnt(8): the 8 loads of the next tile may still be in flight).
 #include "xkv_common.h"
 #include "recon_fast.h"
 #include <type_traits>
 
 namespace xkv {
-
 
 typedef short s16x4f __attribute__((ext_vector_type(4)));
 typedef short s16x8f __attribute__((ext_vector_type(8)));
@@ -37,11 +44,15 @@ constexpr int FROW = 1040;          // LDS bytes per tile row (1024 + 16 pad: 16
 constexpr int FTILE = FT * FROW;    // 33280
 constexpr int FRING = 4;
 constexpr int FSP_ROW = FT + 4;     // partial-score row stride (floats)
+constexpr int FP_ROW = FT + 8;      // P row stride (elements)
+constexpr float LAZY_RESCALE = 16.f; // the softmax reference only moves when a tile maximum exceeds it by this much
 
 // The LDS destination of a direct-to-LDS load is M0 + lane * 16.  A SALU write of M0 needs one wait state
 // before an instruction that reads M0 (the compiler schedules around this for its own code; here it is explicit).
-__device__ __forceinline__ void async_row16(const void* gsrc, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gsrc) : "memory", "m0");
+// Address = scalar row base + per-lane byte offset.
+__device__ __forceinline__ void async_row16(const void* row_base, unsigned lane_off, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_off), "s"(row_base)
+               : "memory", "m0");
 }
 template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
@@ -55,7 +66,7 @@ __global__ __launch_bounds__(256) void pack_b_kernel(const T* __restrict__ kB, T
   const int kh = blockIdx.x, b = blockIdx.y;
   const T* Bh = kB + b * sBb + kh * sBh;
   T* out = Bp + ((int64_t)b * hkv + kh) * (512 * 128);
-  for (int idx = threadIdx.x; idx < 4 * 16 * 2 * 64; idx += 256) {
+  for (int idx = blockIdx.z * 256 + threadIdx.x; idx < 4 * 16 * 2 * 64; idx += 256 * gridDim.z) {
     const int l = idx & 63, blk = (idx >> 6) & 1, ks = (idx >> 7) & 15, w = idx >> 11;
     const int kq = w >> 1, dq = w & 1;
     const int col = 64 * blk + 32 * dq + (l & 31);
@@ -82,8 +93,7 @@ template <bool IS_MAX> __device__ __forceinline__ float row16_reduce(float x) {
   return x;
 }
 
-constexpr int FP_ROW = FT + 8;       // P row stride (elements)
-constexpr float LAZY_RESCALE = 16.f; // the softmax reference only moves when a tile maximum exceeds it by this much
+template <int V> using IC = std::integral_constant<int, V>;
 
 template <typename T>
 __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
@@ -121,16 +131,27 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   if (tid < 16) alpha_lds[tid] = 1.f;
 
   // ---- async tile loads: wave w brings rows 8w .. 8w+7, one 1 KiB row per instruction ------------------------------
-  const unsigned char* Ab = reinterpret_cast<const unsigned char*>(p.kA) + b * p.sAb * 2 + lane * 16;
+  // Scalar row pointers advance by adds only; the clamped form is needed only where a tile crosses the split end.
+  const unsigned char* Ab = reinterpret_cast<const unsigned char*>(p.kA) + b * p.sAb * 2;
   const int64_t row_bytes = p.sAl * 2;
+  const unsigned lane_off = lane * 16;
   auto issue_tile = [&](int t) {
     const unsigned dst = ring_lds + (unsigned)(t & (FRING - 1)) * FTILE + (unsigned)(wave * 8) * FROW;
     const int tok0 = start + t * FT + wave * 8;
+    if (tok0 + 7 <= last) {
+      const unsigned char* row = Ab + (int64_t)tok0 * row_bytes;
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      int tok = tok0 + r;
-      tok = tok < last ? tok : last;   // rows past the split end are masked in the softmax; keep the read in bounds
-      async_row16(Ab + (int64_t)tok * row_bytes, dst + r * FROW);
+      for (int r = 0; r < 8; ++r) {
+        async_row16(row, lane_off, dst + r * FROW);
+        row += row_bytes;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        int tok = tok0 + r;
+        tok = tok < last ? tok : last;   // rows past the split end are masked in the softmax; keep the read in bounds
+        async_row16(Ab + (int64_t)tok * row_bytes, lane_off, dst + r * FROW);
+      }
     }
   };
   issue_tile(0);
@@ -168,30 +189,28 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     }
   }
   const float qinv = p.inv_freq[lane];
-  float qc32, qs32, qcb = 1.f, qsb = 0.f;
+  // q^ is kept in q-dot operand order: pair j = 32 dq' + 8 o + 4 g' + e sits at [o][dq'][g'][e] (partner at e + 4), so that
+  // a lane's 8 contraction values of chunk o are one 16-byte read
+  const int qpos = ((((lane >> 3) & 3) * 2 + (lane >> 5)) * 2 + ((lane >> 2) & 1)) * 8 + (lane & 3);
+  float qc32, qs32, qcb = 1.f, qsb = 0.f;   // (qcb, qsb): base rotation of the tile whose q^ is written next
   sincosf((float)FT * qinv, &qs32, &qc32);
-  auto seed_base = [&](int t) { sincosf((float)(p.pos_offset + start + (int64_t)t * FT) * qinv, &qsb, &qcb); };
-  auto step_base = [&]() {
-    const float c = qcb * qc32 - qsb * qs32, s = qsb * qc32 + qcb * qs32;
-    qcb = c; qsb = s;
-  };
-  auto write_qhat = [&](int t) {   // q^ for tile t = R(-base(t)) q, base held in (qcb, qsb)
-    T* dst = qhat + (t & 1) * (8 * 128) + wave * 128 + lane;
+  auto write_qhat = [&](int t) {   // q^ for tile t = R(-base(t)) q; re-seed the base with a full-range sincos every 32 tiles
+    if ((t & 31) == 0) sincosf((float)(p.pos_offset + start + (int64_t)t * FT) * qinv, &qsb, &qcb);
+    T* dst = qhat + (t & 1) * (8 * 128) + wave * 128 + qpos;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       dst[i * 512] = from_f32<T>(q0[i] * qcb + q1[i] * qsb);
-      dst[i * 512 + 64] = from_f32<T>(q1[i] * qcb - q0[i] * qsb);
+      dst[i * 512 + 4] = from_f32<T>(q1[i] * qcb - q0[i] * qsb);
     }
+    const float c = qcb * qc32 - qsb * qs32, s = qsb * qc32 + qcb * qs32;
+    qcb = c; qsb = s;
   };
 
-  // ---- softmax role: lanes 0..15 of wave w own head w, lanes 16..31 head w + 4; two tokens per lane ---------------------
+  // ---- softmax role: lanes 0..15 of wave w own head w, lanes 16..31 head w + 4 (lanes 32..63 mirror them) --------------
   const int sm_head = wave + 4 * ((lane >> 4) & 1);
   const int sm_row = sm_head < G ? sm_head : G - 1;
-  const bool sm_valid = sm_head < G;   // lanes 32..63 duplicate lanes 0..31 (same values, same addresses)
+  const bool sm_valid = sm_head < G;
   float m_ref = NEG_INF, l_run = 0.f;
-#ifdef XKV_DEBUG_SCORES
-  float dbg0 = 0.f, dbg1 = 0.f;
-#endif
   auto softmax_tile = [&](int t) {   // scores of tile t -> P (operand type) and the rescale factor, through LDS
     const float* sp = s_part + sm_row * FSP_ROW + 2 * n16;
     float s0 = 0.f, s1 = 0.f;
@@ -204,133 +223,193 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     const int tok = start + t * FT + 2 * n16;
     s0 = tok < end ? s0 * p.sm_scale : NEG_INF;
     s1 = tok + 1 < end ? s1 * p.sm_scale : NEG_INF;
-#ifdef XKV_DEBUG_SCORES
-    dbg0 = s0; dbg1 = s1;
-#endif
-    const float mx = row16_reduce<true>(fmaxf(s0, s1));
-    const float m_new = mx > m_ref + LAZY_RESCALE ? mx : m_ref;
-    const float alpha = __expf(m_ref - m_new);
-    const float e0 = __expf(s0 - m_new), e1 = __expf(s1 - m_new);
+    float alpha = 1.f;
+    if (__builtin_amdgcn_ballot_w64(fmaxf(s0, s1) > m_ref + LAZY_RESCALE)) {   // rare after the first tiles
+      const float mx = row16_reduce<true>(fmaxf(s0, s1));
+      const float m_new = mx > m_ref + LAZY_RESCALE ? mx : m_ref;
+      alpha = __expf(m_ref - m_new);
+      m_ref = m_new;
+    }
+    const float e0 = __expf(s0 - m_ref), e1 = __expf(s1 - m_ref);
     l_run = l_run * alpha + row16_reduce<false>(e0 + e1);
-    m_ref = m_new;
     T* pd = p_lds + sm_head * FP_ROW + 2 * n16;
     pd[0] = from_f32<T>(sm_valid ? e0 : 0.f);
     pd[1] = from_f32<T>(sm_valid ? e1 : 0.f);
     alpha_lds[sm_head] = alpha;
   };
 
-  // ---- P.A accumulators: wave w owns latent features 128 w .. +128 -----------------------------------------------------
-  f32x4 acc[8];
+  // ---- accumulators and loop-carried operand registers ---------------------------------------------------------------------
+  f32x4 acc[8];          // P.A: wave w owns latent features 128 w .. +128
 #pragma unroll
   for (int mb = 0; mb < 8; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
-  auto pv_tile = [&](int t) {
-    const float al = alpha_lds[n16];
-    if (__builtin_amdgcn_ballot_w64(al != 1.f)) {   // rare: the softmax reference moved
-#pragma unroll
-      for (int mb = 0; mb < 8; ++mb) acc[mb] *= al;
-    }
-    const vec8 pb = ld16<vec8>(p_lds + n16 * FP_ROW + 8 * g4);
-    const unsigned char* vt = ring + (t & (FRING - 1)) * FTILE + (8 * g4 + (n16 >> 2)) * FROW + (wave * 128 + 4 * (n16 & 3)) * 2;
-#pragma unroll
-    for (int mb = 0; mb < 8; ++mb) {
-      s16x4f a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4f*)(vt + mb * 32));
-      s16x4f a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4f*)(vt + mb * 32 + 4 * FROW));
-      vec8 a = __builtin_bit_cast(vec8, (s16x8f)__builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
-      acc[mb] = Elem<T>::mfma16(a, pb, acc[mb]);
-    }
+  f32x16 ka[2][2];       // two sets of partial key accumulators [set][low | partner feature block]
+  vec8 at[16];           // this wave's 16 rank chunks of the tile being reconstructed (read one part ahead of their use)
+  vec8 qop[4];           // q^ operands of the tile being rotated
+
+  auto tile_frag = [&](int t, int ks) -> vec8 {
+    return ld16<vec8>(ring + (t & (FRING - 1)) * FTILE + n32 * FROW + (256 * kq + 8 * g2) * 2 + ks * 32);
   };
 
-  // ---- reconstruction of this wave's partial key tile, k-steps [KS0, KS1) -----------------------------------------------
-  f32x16 k0, k1;
-  auto recon_steps = [&](int t, auto ks0, auto ks1) {
-    const unsigned char* arow = ring + (t & (FRING - 1)) * FTILE + n32 * FROW + (256 * kq + 8 * g2) * 2;
+  // One pipeline iteration.  PAR: accumulator set written by the reconstruction of tile i; tile i-1 lives in set PAR^1.
+  // Interval structure (two barriers per iteration):
+  //   part 1 [after B_c of i-1]  R(i) k-steps 0..5   ||  rotate tile i-1, q-dot, publish partial scores; write q^(i)
+  //   B_b
+  //   part 2                     R(i) k-steps 6..10  ||  issue tile i+2; softmax of tile i-1; wait for tile i+1
+  //   B_c
+  //   part 3                     R(i) k-steps 11..15 ||  acc += V^T P^T for tile i-1
+  // Every LDS operand is read one part before the MFMAs that consume it.
+  auto iteration = [&](int i, auto par_c, auto do_r_c, auto do_prev_c) {
+    constexpr int PAR = decltype(par_c)::value;
+    constexpr bool DO_R = decltype(do_r_c)::value != 0, DO_PREV = decltype(do_prev_c)::value != 0;
+    f32x16& k0 = ka[PAR][0];
+    f32x16& k1 = ka[PAR][1];
+    const f32x16& j0 = ka[PAR ^ 1][0];
+    const f32x16& j1 = ka[PAR ^ 1][1];
 #pragma unroll
-    for (int ks = decltype(ks0)::value; ks < decltype(ks1)::value; ++ks) {
-      const vec8 at = ld16<vec8>(arow + ks * 32);
-      k0 = Elem<T>::mfma32(breg[ks][0], at, k0);
-      k1 = Elem<T>::mfma32(breg[ks][1], at, k1);
+    for (int ks = 0; ks < 16; ++ks) {
+      asm volatile("" : "+a"(breg[ks][0]));
+      asm volatile("" : "+a"(breg[ks][1]));
     }
-  };
-  // rotate by the in-tile offset, round to the operand type, dot with q^ (4 contraction chunks of 16 features), store
-  auto rope_qdot = [&](int t) {
-    f32x16 sacc;
+    // ---- part 1 ----------------------------------------------------------------------------------------------------------
+    if (DO_R) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
-    const T* qrow = qhat + (t & 1) * (8 * 128) + (n32 < G ? n32 : G - 1) * 128 + 32 * dq + 4 * g2;
+      for (int ks = 6; ks < 11; ++ks) at[ks] = tile_frag(i, ks);
+    }
+    {
+      f32x16 sacc;
 #pragma unroll
-    for (int o = 0; o < 4; ++o) {
-      vec8 kop;
+      for (int o = 0; o < 4; ++o) {
+        if (DO_R) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int r = 4 * o + e;
-        kop[e] = from_f32<T>(k0[r] * ci[r] - k1[r] * si[r]);
-        kop[4 + e] = from_f32<T>(k1[r] * ci[r] + k0[r] * si[r]);
+          for (int m = 3 * o; m < 3 * o + 3; ++m) {
+            const int ks = m >> 1;
+            if (ks == 0) {
+              const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+              if ((m & 1) == 0) k0 = Elem<T>::mfma32(breg[0][0], at[0], z); else k1 = Elem<T>::mfma32(breg[0][1], at[0], z);
+            } else {
+              if ((m & 1) == 0) k0 = Elem<T>::mfma32(breg[ks][0], at[ks], k0); else k1 = Elem<T>::mfma32(breg[ks][1], at[ks], k1);
+            }
+          }
+        }
+        if (DO_PREV) {
+          vec8 kop;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int r = 4 * o + e;
+            kop[e] = from_f32<T>(j0[r] * ci[r] - j1[r] * si[r]);
+            kop[4 + e] = from_f32<T>(j1[r] * ci[r] + j0[r] * si[r]);
+          }
+          if (o == 0) {
+            const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            sacc = Elem<T>::mfma32(kop, qop[o], z);
+          } else {
+            sacc = Elem<T>::mfma32(kop, qop[o], sacc);
+          }
+        }
       }
-      const u32x2 ql = *reinterpret_cast<const u32x2*>(qrow + 8 * o);
-      const u32x2 qh = *reinterpret_cast<const u32x2*>(qrow + 64 + 8 * o);
-      const u32x4 qq = {ql[0], ql[1], qh[0], qh[1]};
-      sacc = Elem<T>::mfma32(kop, __builtin_bit_cast(vec8, qq), sacc);
-    }
-    // lane (n32 = head, g2): register r = token 8 (r/4) + 4 g2 + r%4
-    if (n32 < G) {
-      float* dst = s_part + (wave * 8 + n32) * FSP_ROW + 4 * g2;
+      if (DO_R) write_qhat(i);
+      // lane (n32 = head, g2): register r of sacc = token 8 (r/4) + 4 g2 + r%4
+      if (DO_PREV && n32 < G) {
+        float* dst = s_part + (wave * 8 + n32) * FSP_ROW + 4 * g2;
 #pragma unroll
-      for (int qd = 0; qd < 4; ++qd)
-        *reinterpret_cast<f32x4*>(dst + 8 * qd) = f32x4{sacc[4 * qd], sacc[4 * qd + 1], sacc[4 * qd + 2], sacc[4 * qd + 3]};
+        for (int qd = 0; qd < 4; ++qd)
+          *reinterpret_cast<f32x4*>(dst + 8 * qd) = f32x4{sacc[4 * qd], sacc[4 * qd + 1], sacc[4 * qd + 2], sacc[4 * qd + 3]};
+      }
+    }
+    __syncthreads();        // B_b: partial scores of tile i-1 and q^(i) are visible; every wave is past P.A of tile i-2
+    // ---- part 2 ----------------------------------------------------------------------------------------------------------
+    s16x4f tr[16];
+    if (DO_R) {
+#pragma unroll
+      for (int ks = 11; ks < 16; ++ks) at[ks] = tile_frag(i, ks);
+    }
+    if (DO_PREV) {
+      const unsigned char* vt =
+          ring + ((i - 1) & (FRING - 1)) * FTILE + (8 * g4 + (n16 >> 2)) * FROW + (wave * 128 + 4 * (n16 & 3)) * 2;
+#pragma unroll
+      for (int mb = 0; mb < 8; ++mb) {
+        tr[2 * mb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4f*)(vt + mb * 32));
+        tr[2 * mb + 1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4f*)(vt + mb * 32 + 4 * FROW));
+      }
+    }
+    if (DO_R) {
+      k0 = Elem<T>::mfma32(breg[6][0], at[6], k0);
+      k1 = Elem<T>::mfma32(breg[6][1], at[6], k1);
+      issue_tile(i + 2);    // its ring slot was last read by the P.A of tile i-2, finished before B_b
+      k0 = Elem<T>::mfma32(breg[7][0], at[7], k0);
+      k1 = Elem<T>::mfma32(breg[7][1], at[7], k1);
+    }
+    if (DO_PREV) softmax_tile(i - 1);
+    if (DO_R) {
+#pragma unroll
+      for (int ks = 8; ks < 11; ++ks) {
+        k0 = Elem<T>::mfma32(breg[ks][0], at[ks], k0);
+        k1 = Elem<T>::mfma32(breg[ks][1], at[ks], k1);
+      }
+      wait_vmcnt<8>();      // this wave's rows of tile i+1 have landed (the 8 loads of tile i+2 may be in flight)
+    } else {
+      wait_vmcnt<0>();
+      if (sm_valid && n16 == 0) { ml_lds[2 * sm_head] = m_ref; ml_lds[2 * sm_head + 1] = l_run; }   // final state for the epilogue
+    }
+    __syncthreads();        // B_c: P and rescale factors of tile i-1 are visible; tile i+1 is complete for every wave
+    // ---- part 3 ----------------------------------------------------------------------------------------------------------
+    vec8 pb;
+    if (DO_PREV) {
+      const float al = alpha_lds[n16];
+      pb = ld16<vec8>(p_lds + n16 * FP_ROW + 8 * g4);
+      if (__builtin_amdgcn_ballot_w64(al != 1.f)) {   // rare: the softmax reference moved
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) acc[mb] *= al;
+      }
+    }
+    vec8 at_next[6], qop_next[4];
+    if (DO_R) {
+#pragma unroll
+      for (int ks = 0; ks < 6; ++ks) at_next[ks] = tile_frag(i + 1, ks);
+      const T* qrow = qhat + (i & 1) * (8 * 128) + (n32 < G ? n32 : G - 1) * 128 + (dq * 2 + g2) * 8;
+#pragma unroll
+      for (int o = 0; o < 4; ++o) qop_next[o] = ld16<vec8>(qrow + o * 32);
+    }
+#pragma unroll
+    for (int u = 0; u < 5; ++u) {
+      if (DO_R) {
+        k0 = Elem<T>::mfma32(breg[11 + u][0], at[11 + u], k0);
+        k1 = Elem<T>::mfma32(breg[11 + u][1], at[11 + u], k1);
+      }
+      if (DO_PREV) {
+#pragma unroll
+        for (int mb = (u * 8) / 5; mb < ((u + 1) * 8) / 5; ++mb) {
+          vec8 a = __builtin_bit_cast(vec8, (s16x8f)__builtin_shufflevector(tr[2 * mb], tr[2 * mb + 1], 0, 1, 2, 3, 4, 5, 6, 7));
+          acc[mb] = Elem<T>::mfma16(a, pb, acc[mb]);
+        }
+      }
+    }
+    if (DO_R) {
+#pragma unroll
+      for (int ks = 0; ks < 6; ++ks) at[ks] = at_next[ks];
+#pragma unroll
+      for (int o = 0; o < 4; ++o) qop[o] = qop_next[o];
     }
   };
-  auto zero_k = [&]() {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) { k0[r] = 0.f; k1[r] = 0.f; }
-  };
-  typedef std::integral_constant<int, 0> I0;
-  typedef std::integral_constant<int, 8> I8;
-  typedef std::integral_constant<int, 16> I16;
 
-  // ---- tile 0: no predecessor to finish ---------------------------------------------------------------------------------
-  seed_base(0);
-  write_qhat(0);
-  step_base();              // (qcb, qsb) always holds the base of the next tile whose q^ is to be written
-  wait_vmcnt<8>();
+  // ---- pipeline: R(0) | {R(i), prev(i-1)} for i = 1 .. ntiles-1 | prev(ntiles-1) -------------------------------------------------
+  wait_vmcnt<8>();          // tile 0 (tile 1 may be in flight)
   __syncthreads();
-  issue_tile(2);
-  zero_k();
-  recon_steps(0, I0(), I16());
-  rope_qdot(0);
-
-  // ---- steady state: tile t is reconstructed while tile t-1 goes through softmax and P.A ------------------------------------
-  int t = 1;
-  while (t < ntiles) {
-    const int chunk_end = (t | 31) + 1 < ntiles ? (t | 31) + 1 : ntiles;
-    if ((t & 31) == 0) seed_base(t);   // re-seed the base angle with a full-range sincos every 32 tiles
-    for (; t < chunk_end; ++t) {
 #pragma unroll
-      for (int ks = 0; ks < 16; ++ks) {
-#ifndef XKV_NO_PIN
-        asm volatile("" : "+a"(breg[ks][0]));
-        asm volatile("" : "+a"(breg[ks][1]));
-#endif
-      }
-      wait_vmcnt<8>();        // this wave's rows of tile t have landed (tile t+1's 8 loads may be in flight)
-      __syncthreads();        // B1: tile t and the partial scores of tile t-1 are complete for every wave
-      issue_tile(t + 2);
-      write_qhat(t);
-      step_base();
-      zero_k();
-      softmax_tile(t - 1);
-      recon_steps(t, I0(), I8());
-      __syncthreads();        // B2: P and the rescale factors of tile t-1 are visible
-      recon_steps(t, I8(), I16());
-      pv_tile(t - 1);
-      rope_qdot(t);
-    }
+  for (int ks = 0; ks < 6; ++ks) at[ks] = tile_frag(0, ks);
+  iteration(0, IC<0>(), IC<1>(), IC<0>());
+  int i = 1;
+  for (; i + 1 < ntiles; i += 2) {
+    iteration(i, IC<1>(), IC<1>(), IC<1>());
+    iteration(i + 1, IC<0>(), IC<1>(), IC<1>());
   }
-  wait_vmcnt<0>();
+  if (i < ntiles) {
+    iteration(i, IC<1>(), IC<1>(), IC<1>());
+    ++i;
+  }
+  if (ntiles & 1) iteration(ntiles, IC<1>(), IC<0>(), IC<1>());
+  else iteration(ntiles, IC<0>(), IC<0>(), IC<1>());
   __syncthreads();
-  softmax_tile(ntiles - 1);
-  if (sm_valid && n16 == 0) { ml_lds[2 * sm_head] = m_ref; ml_lds[2 * sm_head + 1] = l_run; }
-  __syncthreads();
-  pv_tile(ntiles - 1);
 
   // ---- epilogue ----------------------------------------------------------------------------------------------------------
   if (n16 < G) {
@@ -342,13 +421,6 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     for (int mb = 0; mb < 8; ++mb) *reinterpret_cast<f32x4*>(dst + mb * 16) = acc[mb] * inv;
     if (wave == 0 && g4 == 0) p.lse[ph] = m + __logf(l);
   }
-#ifdef XKV_DEBUG_SCORES
-  __syncthreads();
-  if (sm_valid && lane < 16) {   // last tile's scaled scores of head sm_head into the first 32 partial columns
-    float* dst = p.partial + (((int64_t)b * p.hq + h0 + sm_head) * p.max_splits + split) * 512 + 2 * n16;
-    dst[0] = dbg0; dst[1] = dbg1;
-  }
-#endif
 }
 
 constexpr size_t FAST_SHM = (size_t)FRING * FTILE + 4 * 8 * FSP_ROW * 4 + 2 * 8 * 128 * 2 + 16 * FP_ROW * 2 + 16 * 4 + 16 * 4;
@@ -356,7 +428,7 @@ constexpr size_t FAST_SHM = (size_t)FRING * FTILE + 4 * 8 * FSP_ROW * 4 + 2 * 8 
 template <typename T>
 int launch_recon_fast_t(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, hipStream_t st) {
   const int nb = sBb == 0 ? 1 : batch;   // one packed copy when the factor is shared by the batch
-  pack_b_kernel<T><<<dim3(p.hkv, nb), dim3(256), 0, st>>>((const T*)kB, (T*)p.Bp, sBb, sBh, sBr, p.hkv);
+  pack_b_kernel<T><<<dim3(p.hkv, nb, 32), dim3(256), 0, st>>>((const T*)kB, (T*)p.Bp, sBb, sBh, sBr, p.hkv);
   auto kern = recon_fast_kernel<T>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)FAST_SHM);
