@@ -76,6 +76,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     const int32_t* __restrict__ num_kv_splits, const int32_t* __restrict__ kv_lens,
     int hq, int hkv, int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh) {
   extern __shared__ float merged[];  // [G][dv]
+  __shared__ float fin[4 * 256];     // per-head-block totals of the up-projection
   const int kh = blockIdx.x, b = blockIdx.y, G = hq / hkv;
   const int L = kv_lens ? kv_lens[b] : kv_len;
   const int ns = num_kv_splits[b];
@@ -107,26 +108,60 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
   }
   if (!vB) return;
   __syncthreads();
+  // out[g][c] = sum_rho merged[g][rho] * vB[rho][c].  Thread -> (8 output columns, one of 256/ncb rank groups): 16-byte
+  // loads of vB, several in flight, then a reduction over the rank groups through LDS.
+  typedef typename Elem<TB>::vec8 vec8;
   const TB* Bh = vB + b * sVb + kh * sVh;
-  // thread -> (output column, rank slice); slices reduced through LDS atomics-free tree
-  const int nsl = blockDim.x / d_out;  // d_out <= 256 -> nsl >= 1
-  const int col = threadIdx.x % d_out, sl = threadIdx.x / d_out;
-  __shared__ float red[256 * 16];
-  float acc[16];
-  for (int gi = 0; gi < G; ++gi) acc[gi] = 0.f;
-  if (sl < nsl) {
-    for (int rho = sl; rho < dv; rho += nsl) {
-      float w = to_f32(Bh[rho * sVr + col]);
-      for (int gi = 0; gi < G; ++gi) acc[gi] += merged[gi * dv + rho] * w;
+  __shared__ float red[32 * 4 * 64];                 // [rank group][4 heads][columns of the block]  (<= 32 KiB)
+  const int ncb = (d_out + 7) >> 3;                  // 8-column blocks (d_out <= 256 -> <= 32)
+  const int ngrp = 256 / ncb;                        // rank groups
+  const int cb = threadIdx.x % ncb, grp = threadIdx.x / ncb;
+  const bool active = grp < ngrp && cb * 8 + 8 <= d_out;
+  for (int g0 = 0; g0 < G; g0 += 4) {
+    float acc[4][8];
+#pragma unroll
+    for (int gi = 0; gi < 4; ++gi)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[gi][e] = 0.f;
+    if (active) {
+#pragma unroll 4
+      for (int rho = grp; rho < dv; rho += ngrp) {
+        const vec8 w = ld16<vec8>(Bh + rho * sVr + cb * 8);
+#pragma unroll
+        for (int gi = 0; gi < 4; ++gi) {
+          const float m = g0 + gi < G ? merged[(g0 + gi) * dv + rho] : 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[gi][e] += m * to_f32(w[e]);
+        }
+      }
     }
-  }
-  for (int gi = 0; gi < G; ++gi) red[gi * 256 + threadIdx.x] = (sl < nsl) ? acc[gi] : 0.f;
-  __syncthreads();
-  for (int idx = threadIdx.x; idx < G * d_out; idx += blockDim.x) {
-    const int gi = idx / d_out, c = idx - gi * d_out;
-    float s = 0.f;
-    for (int k = 0; k < nsl; ++k) s += red[gi * 256 + k * d_out + c];
-    out[b * sOb + (kh * G + gi) * sOh + c] = (O)s;
+    // reduce over the rank groups through LDS, `chunk` groups per pass (as many as fit `red`)
+    const int cols = ncb * 8;                        // <= 256
+    const int chunk = 32 * 64 / cols;                // >= 8
+    for (int base = 0; base < ngrp; base += chunk) {
+      __syncthreads();
+      if (active && grp >= base && grp < base + chunk) {
+#pragma unroll
+        for (int gi = 0; gi < 4; ++gi)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) red[((grp - base) * 4 + gi) * cols + cb * 8 + e] = acc[gi][e];
+      }
+      __syncthreads();
+      const int n_here = (ngrp - base) < chunk ? (ngrp - base) : chunk;
+      for (int idx = threadIdx.x; idx < 4 * d_out; idx += blockDim.x) {
+        const int gi = idx / d_out, c = idx - gi * d_out;
+        if (g0 + gi < G) {
+          float sacc = 0.f;
+          for (int k = 0; k < n_here; ++k) sacc += red[(k * 4 + gi) * cols + c];
+          fin[idx] = (base == 0 ? 0.f : fin[idx]) + sacc;
+        }
+      }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 4 * d_out; idx += blockDim.x) {
+      const int gi = idx / d_out, c = idx - gi * d_out;
+      if (g0 + gi < G) out[b * sOb + (kh * G + g0 + gi) * sOh + c] = (O)fin[idx];
+    }
   }
 }
 
@@ -205,7 +240,7 @@ extern "C" int xkv_merge_stage2(const float* partial, const float* lse, void* ou
   if (!partial || !lse || !out || !ns || batch <= 0 || hq <= 0 || hkv <= 0 || max_splits <= 0 || dv <= 0)
     return XKV_EINVAL;
   if (hq % hkv || hq / hkv > 16 || dv > 512) return XKV_EUNSUPPORTED;
-  if (vB && (d_out <= 0 || d_out > 256)) return XKV_EUNSUPPORTED;
+  if (vB && (d_out <= 0 || d_out > 256 || d_out % 8)) return XKV_EUNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
 #define XKV_MERGE(O, TB) \
   return launch_merge<O, TB>(partial, lse, out, vB, sVb, sVh, sVr, d_out, ns, kl, batch, hq, hkv, kv_len, max_splits, dv, sOb, sOh, st)
