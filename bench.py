@@ -122,7 +122,7 @@ def bench_c3(args, dev):
         "tokens_per_s": B / (us * 1e-6), "kv_tokens_scanned_per_s": B * L / (us * 1e-6),
         "config": {"workload": "c3 fused RoPE xKV decode: batch 16, 32q/8kv heads, d128, ctx %d, rank 512, "
                                "A shared by K/V and by a 4-layer group, per layer" % L, "kv_splits": S},
-        "roofline": {"bound": "mfma", "kernel": "recon_stage1_kernel", "achieved": round(achieved, 1),
+        "roofline": {"bound": "mfma", "kernel": "recon_fast_kernel", "achieved": round(achieved, 1),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                      "traffic": None, "kernel_avg_us": round(k_avg_ms * 1e3, 2), "kernel_median_us": round(k_med_ms * 1e3, 2),
                      "algorithmic_flop": flops, "hbm_side_GBps": round(algo_bytes / (k_avg_ms * 1e-3) / 1e9, 1)},
@@ -279,6 +279,9 @@ def main():
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-comparator", action="store_true")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run 3 plain device copies of 512 MiB (a kernel of known traffic, for scaling rocprof's "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -286,6 +289,13 @@ def main():
     _lib.lib()  # fail loudly if the HIP library is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calib_copy:
+        src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if args.config == "c3":
         res = bench_c3(args, dev)
     elif args.config == "c2":
