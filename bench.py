@@ -25,6 +25,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBS = 8000.0
 PEAK_BF16_TFLOPS = 2500.0
+# HBM bytes of one stage-1 launch at the default c3 shape, from two rocprofv3 --pmc runs of this file
+# (FETCH_SIZE, WRITE_SIZE; each scaled by what the counter reads for --calib-copy's 512 MiB copies).
+# A counter cannot be read from inside the timed process, so the figure is recorded here.
+C3_STAGE1_HBM_BYTES = 535259 * 1024
 
 
 def _events(n):
@@ -124,7 +128,8 @@ def bench_c3(args, dev):
                                "A shared by K/V and by a 4-layer group, per layer" % L, "kv_splits": S},
         "roofline": {"bound": "mfma", "kernel": "recon_fast_kernel", "achieved": round(achieved, 1),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-                     "traffic": None, "kernel_avg_us": round(k_avg_ms * 1e3, 2), "kernel_median_us": round(k_med_ms * 1e3, 2),
+                     "traffic": C3_STAGE1_HBM_BYTES if (L == 32768 and not args.splits) else None,
+                     "kernel_avg_us": round(k_avg_ms * 1e3, 2), "kernel_median_us": round(k_med_ms * 1e3, 2),
                      "algorithmic_flop": flops, "hbm_side_GBps": round(algo_bytes / (k_avg_ms * 1e-3) / 1e9, 1)},
         "uncompressed_flash_decode_us": None if comp_us is None else round(comp_us, 2),
         "cpu_baseline": cpu,

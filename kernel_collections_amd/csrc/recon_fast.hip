@@ -16,12 +16,14 @@
 // and read back as the B operand of the q-dot MFMA.
 //
 // Pipeline.  A wave issues instructions in order, so MFMA time and VALU time only overlap when independent
-// work is interleaved in its instruction stream.  Iteration i therefore runs the reconstruction MFMAs of tile i
-// (accumulating into one of two key-accumulator sets) in three parts, interleaved with what tile i-1 still
-// needs: part 1 rotates tile i-1's partial keys (the other accumulator set) and dots them with q^; part 2 runs
-// the softmax of tile i-1 (wave w owns head w and w+4: no redundant work) and publishes P and the rescale
-// factor through LDS; part 3 accumulates P.A for tile i-1, each wave owning 128 latent features, the token-
-// major operand coming from ds_read_b64_tr_b16.  Three balanced barriers per tile separate the parts.
+// work is interleaved in its instruction stream.  Iteration i therefore runs the 16 reconstruction MFMA steps of
+// tile i (accumulating into one of two key-accumulator sets) in three parts, interleaved with what tile i-1 still
+// needs: part 1 (steps 0..5) rotates tile i-1's partial keys (the other accumulator set), dots them with q^ and
+// stores the partial scores, while the pair-index threads write q^ for tile i; barrier; part 2 (steps 6..10)
+// issues the loads of tile i+2, runs the softmax of tile i-1 (one owner lane group per head: no redundant work)
+// and publishes P and the rescale factor through LDS; barrier; part 3 (steps 11..15) accumulates P.A for tile
+// i-1, each wave owning 128 latent features, the token-major operand coming from ds_read_b64_tr_b16, and
+// prefetches the first LDS operands of tile i+1.  Two barriers per tile separate the parts.
 // The softmax reference only moves when a tile maximum exceeds it by 16 (lazy rescaling), so the P.A
 // accumulators are almost never rescaled.
 //
