@@ -18,6 +18,12 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-inline-asm",
 ]
+# Per-file additions.  recon_fast.hip: MFMA results must land in ordinary VGPRs (the RoPE / softmax VALU code reads
+# them; with accumulation-register results every value costs a v_accvgpr_read), while the stationary B operands are
+# pinned to accumulation registers by the source itself.
+EXTRA_FLAGS = {
+    "recon_fast.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
 
 
 def sources():
@@ -26,7 +32,7 @@ def sources():
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ, src[:-4] + ".o")
-    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC, *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
