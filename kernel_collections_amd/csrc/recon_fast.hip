@@ -137,10 +137,10 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   const unsigned char* Ab = reinterpret_cast<const unsigned char*>(p.kA) + b * p.sAb * 2;
   const int64_t row_bytes = p.sAl * 2;
   const unsigned lane_off = lane * 16;
-  auto issue_tile = [&](int t) {
+  auto issue_tile = [&](int t, auto full_c) {
     const unsigned dst = ring_lds + (unsigned)(t & (FRING - 1)) * FTILE + (unsigned)(wave * 8) * FROW;
     const int tok0 = start + t * FT + wave * 8;
-    if (tok0 + 7 <= last) {
+    if (decltype(full_c)::value || tok0 + 7 <= last) {   // full_c: the caller knows the whole tile lies inside the split
       const unsigned char* row = Ab + (int64_t)tok0 * row_bytes;
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
@@ -156,8 +156,9 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       }
     }
   };
-  issue_tile(0);
-  issue_tile(1);
+  issue_tile(0, IC<0>());
+  issue_tile(1, IC<0>());
+  issue_tile(2, IC<0>());
 
   // ---- stationary B operands: 16 k-steps x 2 feature blocks, kept in accumulation registers ---------------------------
   vec8 breg[16][2];
@@ -196,8 +197,18 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   const int qpos = ((((lane >> 3) & 3) * 2 + (lane >> 5)) * 2 + ((lane >> 2) & 1)) * 8 + (lane & 3);
   float qc32, qs32, qcb = 1.f, qsb = 0.f;   // (qcb, qsb): base rotation of the tile whose q^ is written next
   sincosf((float)FT * qinv, &qs32, &qc32);
-  auto write_qhat = [&](int t) {   // q^ for tile t = R(-base(t)) q; re-seed the base with a full-range sincos every 32 tiles
-    if ((t & 31) == 0) sincosf((float)(p.pos_offset + start + (int64_t)t * FT) * qinv, &qsb, &qcb);
+  // The base advances by angle addition; every 32 tiles it is replaced by a freshly range-reduced value (the seed),
+  // computed outside the pipeline's inner loop and swapped in with a select so that write_qhat stays branch-free.
+  int seed_t = 0;
+  float seed_c, seed_s;
+  auto make_seed = [&](int t) {
+    seed_t = t;
+    sincosf((float)(p.pos_offset + start + (int64_t)t * FT) * qinv, &seed_s, &seed_c);
+  };
+  auto write_qhat = [&](int t) {   // q^ for tile t = R(-base(t)) q
+    const bool sd = t == seed_t;
+    qcb = sd ? seed_c : qcb;
+    qsb = sd ? seed_s : qsb;
     T* dst = qhat + (t & 1) * (8 * 128) + wave * 128 + qpos;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -207,6 +218,8 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     const float c = qcb * qc32 - qsb * qs32, s = qsb * qc32 + qcb * qs32;
     qcb = c; qsb = s;
   };
+  make_seed(0);
+  write_qhat(0);
 
   // ---- softmax role: lanes 0..15 of wave w own head w, lanes 16..31 head w + 4 (lanes 32..63 mirror them) --------------
   const int sm_head = wave + 4 * ((lane >> 4) & 1);
@@ -254,13 +267,13 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
 
   // One pipeline iteration.  PAR: accumulator set written by the reconstruction of tile i; tile i-1 lives in set PAR^1.
   // Interval structure (two barriers per iteration):
-  //   part 1 [after B_c of i-1]  R(i) k-steps 0..5   ||  rotate tile i-1, q-dot, publish partial scores; write q^(i)
+  //   part 1 [after B_c of i-1]  R(i) k-steps 0..5   ||  rotate tile i-1, q-dot, publish partial scores
   //   B_b
-  //   part 2                     R(i) k-steps 6..10  ||  issue tile i+2; softmax of tile i-1; wait for tile i+1
+  //   part 2                     R(i) k-steps 6..10  ||  softmax of tile i-1; wait for tile i+1
   //   B_c
-  //   part 3                     R(i) k-steps 11..15 ||  acc += V^T P^T for tile i-1
-  // Every LDS operand is read one part before the MFMAs that consume it.
-  auto iteration = [&](int i, auto par_c, auto do_r_c, auto do_prev_c) {
+  //   part 3                     R(i) k-steps 11..15 ||  acc += V^T P^T for tile i-1; issue tile i+3; write q^(i+1)
+  // Every LDS operand is read one part before the MFMAs that consume it.  FULL: tile i+3 lies wholly inside the split.
+  auto iteration = [&](int i, auto par_c, auto do_r_c, auto do_prev_c, auto full_c) {
     constexpr int PAR = decltype(par_c)::value;
     constexpr bool DO_R = decltype(do_r_c)::value != 0, DO_PREV = decltype(do_prev_c)::value != 0;
     f32x16& k0 = ka[PAR][0];
@@ -309,7 +322,6 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
           }
         }
       }
-      if (DO_R) write_qhat(i);
       // lane (n32 = head, g2): register r of sacc = token 8 (r/4) + 4 g2 + r%4
       if (DO_PREV && n32 < G) {
         float* dst = s_part + (wave * 8 + n32) * FSP_ROW + 4 * g2;
@@ -318,7 +330,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
           *reinterpret_cast<f32x4*>(dst + 8 * qd) = f32x4{sacc[4 * qd], sacc[4 * qd + 1], sacc[4 * qd + 2], sacc[4 * qd + 3]};
       }
     }
-    __syncthreads();        // B_b: partial scores of tile i-1 and q^(i) are visible; every wave is past P.A of tile i-2
+    __syncthreads();        // B_b: partial scores of tile i-1 are visible
     // ---- part 2 ----------------------------------------------------------------------------------------------------------
     s16x4f tr[16];
     if (DO_R) {
@@ -337,7 +349,6 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     if (DO_R) {
       k0 = Elem<T>::mfma32(breg[6][0], at[6], k0);
       k1 = Elem<T>::mfma32(breg[6][1], at[6], k1);
-      issue_tile(i + 2);    // its ring slot was last read by the P.A of tile i-2, finished before B_b
       k0 = Elem<T>::mfma32(breg[7][0], at[7], k0);
       k1 = Elem<T>::mfma32(breg[7][1], at[7], k1);
     }
@@ -353,7 +364,8 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       wait_vmcnt<0>();
       if (sm_valid && n16 == 0) { ml_lds[2 * sm_head] = m_ref; ml_lds[2 * sm_head + 1] = l_run; }   // final state for the epilogue
     }
-    __syncthreads();        // B_c: P and rescale factors of tile i-1 are visible; tile i+1 is complete for every wave
+    __syncthreads();        // B_c: P and rescale factors of tile i-1 are visible; tile i+1 is complete for every wave;
+                            // the transposed reads of tile i-1 have returned, so its ring slot is free
     // ---- part 3 ----------------------------------------------------------------------------------------------------------
     vec8 pb;
     if (DO_PREV) {
@@ -377,6 +389,8 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       if (DO_R) {
         k0 = Elem<T>::mfma32(breg[11 + u][0], at[11 + u], k0);
         k1 = Elem<T>::mfma32(breg[11 + u][1], at[11 + u], k1);
+        if (u == 0) issue_tile(i + 3, full_c);   // into the slot of tile i-1
+        if (u == 2) write_qhat(i + 1);           // buffer (i+1)&1 was last read in part 3 of iteration i-1
       }
       if (DO_PREV) {
 #pragma unroll
@@ -395,22 +409,31 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   };
 
   // ---- pipeline: R(0) | {R(i), prev(i-1)} for i = 1 .. ntiles-1 | prev(ntiles-1) -------------------------------------------------
-  wait_vmcnt<8>();          // tile 0 (tile 1 may be in flight)
+  wait_vmcnt<0>();          // tiles 0..2 and the B operands
   __syncthreads();
 #pragma unroll
   for (int ks = 0; ks < 6; ++ks) at[ks] = tile_frag(0, ks);
-  iteration(0, IC<0>(), IC<1>(), IC<0>());
+  const int nfull = (end - start) / FT;
+  iteration(0, IC<0>(), IC<1>(), IC<0>(), IC<0>());
   int i = 1;
-  for (; i + 1 < ntiles; i += 2) {
-    iteration(i, IC<1>(), IC<1>(), IC<1>());
-    iteration(i + 1, IC<0>(), IC<1>(), IC<1>());
-  }
+  // pairs of iterations in chunks that end where q^ is re-seeded; `fast` pairs know that tiles i+3 and i+4 are full
+  auto pairs = [&](auto full_c) {
+    while (i + 1 < ntiles && (!decltype(full_c)::value || i + 5 <= nfull)) {
+      make_seed((i + 32) & ~31);
+      for (; i < seed_t && i + 1 < ntiles && (!decltype(full_c)::value || i + 5 <= nfull); i += 2) {
+        iteration(i, IC<1>(), IC<1>(), IC<1>(), full_c);
+        iteration(i + 1, IC<0>(), IC<1>(), IC<1>(), full_c);
+      }
+    }
+  };
+  pairs(IC<1>());
+  pairs(IC<0>());
   if (i < ntiles) {
-    iteration(i, IC<1>(), IC<1>(), IC<1>());
+    iteration(i, IC<1>(), IC<1>(), IC<1>(), IC<0>());
     ++i;
   }
-  if (ntiles & 1) iteration(ntiles, IC<1>(), IC<0>(), IC<1>());
-  else iteration(ntiles, IC<0>(), IC<0>(), IC<1>());
+  if (ntiles & 1) iteration(ntiles, IC<1>(), IC<0>(), IC<1>(), IC<0>());
+  else iteration(ntiles, IC<0>(), IC<0>(), IC<1>(), IC<0>());
   __syncthreads();
 
   // ---- epilogue ----------------------------------------------------------------------------------------------------------
