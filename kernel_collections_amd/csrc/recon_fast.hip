@@ -96,6 +96,8 @@ template <bool IS_MAX> __device__ __forceinline__ float row16_reduce(float x) {
 }
 
 template <int V> using IC = std::integral_constant<int, V>;
+#define XKV_FENCE() __builtin_amdgcn_sched_barrier(0)
+#define XKV_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)   // 0x8 MFMA, 0x2 VALU, 0x100 LDS read, 0x200 LDS write
 
 template <typename T>
 __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
@@ -137,25 +139,27 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   const unsigned char* Ab = reinterpret_cast<const unsigned char*>(p.kA) + b * p.sAb * 2;
   const int64_t row_bytes = p.sAl * 2;
   const unsigned lane_off = lane * 16;
-  auto issue_tile = [&](int t, auto full_c) {
+  auto issue_rows = [&](int t, auto r0_c, auto r1_c, auto full_c) {   // rows r0 .. r1-1 of this wave's 8 rows of tile t
+    constexpr int R0 = decltype(r0_c)::value, R1 = decltype(r1_c)::value;
     const unsigned dst = ring_lds + (unsigned)(t & (FRING - 1)) * FTILE + (unsigned)(wave * 8) * FROW;
     const int tok0 = start + t * FT + wave * 8;
-    if (decltype(full_c)::value || tok0 + 7 <= last) {   // full_c: the caller knows the whole tile lies inside the split
-      const unsigned char* row = Ab + (int64_t)tok0 * row_bytes;
+    if (decltype(full_c)::value) {   // the caller knows the whole tile lies inside the split
+      const unsigned char* row = Ab + (int64_t)(tok0 + R0) * row_bytes;
 #pragma unroll
-      for (int r = 0; r < 8; ++r) {
+      for (int r = R0; r < R1; ++r) {
         async_row16(row, lane_off, dst + r * FROW);
         row += row_bytes;
       }
     } else {
 #pragma unroll
-      for (int r = 0; r < 8; ++r) {
+      for (int r = R0; r < R1; ++r) {
         int tok = tok0 + r;
         tok = tok < last ? tok : last;   // rows past the split end are masked in the softmax; keep the read in bounds
         async_row16(Ab + (int64_t)tok * row_bytes, lane_off, dst + r * FROW);
       }
     }
   };
+  auto issue_tile = [&](int t, auto full_c) { issue_rows(t, IC<0>(), IC<8>(), full_c); };
   issue_tile(0, IC<0>());
   issue_tile(1, IC<0>());
   issue_tile(2, IC<0>());
@@ -226,25 +230,23 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   const int sm_row = sm_head < G ? sm_head : G - 1;
   const bool sm_valid = sm_head < G;
   float m_ref = NEG_INF, l_run = 0.f;
-  auto softmax_tile = [&](int t) {   // scores of tile t -> P (operand type) and the rescale factor, through LDS
+  f32x2 sp_v[4];
+  auto softmax_read = [&]() {   // the four waves' partial scores of this lane's two tokens
     const float* sp = s_part + sm_row * FSP_ROW + 2 * n16;
-    float s0 = 0.f, s1 = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const f32x2 v = *reinterpret_cast<const f32x2*>(sp + w * 8 * FSP_ROW);
-      s0 += v[0];
-      s1 += v[1];
-    }
+    for (int w = 0; w < 4; ++w) sp_v[w] = *reinterpret_cast<const f32x2*>(sp + w * 8 * FSP_ROW);
+  };
+  auto softmax_tile = [&](int t) {   // scores of tile t -> P (operand type) and the rescale factor, through LDS
+    float s0 = (sp_v[0][0] + sp_v[1][0]) + (sp_v[2][0] + sp_v[3][0]);
+    float s1 = (sp_v[0][1] + sp_v[1][1]) + (sp_v[2][1] + sp_v[3][1]);
     const int tok = start + t * FT + 2 * n16;
     s0 = tok < end ? s0 * p.sm_scale : NEG_INF;
     s1 = tok + 1 < end ? s1 * p.sm_scale : NEG_INF;
-    float alpha = 1.f;
-    if (__builtin_amdgcn_ballot_w64(fmaxf(s0, s1) > m_ref + LAZY_RESCALE)) {   // rare after the first tiles
-      const float mx = row16_reduce<true>(fmaxf(s0, s1));
-      const float m_new = mx > m_ref + LAZY_RESCALE ? mx : m_ref;
-      alpha = __expf(m_ref - m_new);
-      m_ref = m_new;
-    }
+    // the reference maximum only moves when the tile maximum exceeds it by LAZY_RESCALE (branch-free: alpha = 1 otherwise)
+    const float mx = row16_reduce<true>(fmaxf(s0, s1));
+    const float m_new = mx > m_ref + LAZY_RESCALE ? mx : m_ref;
+    const float alpha = __expf(m_ref - m_new);
+    m_ref = m_new;
     const float e0 = __expf(s0 - m_ref), e1 = __expf(s1 - m_ref);
     l_run = l_run * alpha + row16_reduce<false>(e0 + e1);
     T* pd = p_lds + sm_head * FP_ROW + 2 * n16;
@@ -285,16 +287,17 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       asm volatile("" : "+a"(breg[ks][0]));
       asm volatile("" : "+a"(breg[ks][1]));
     }
+    // Groups of instructions between XKV_FENCE() are scheduled by the compiler on their own and stay in source order:
+    // LDS reads and the tile loads are dealt out among the MFMAs instead of being hoisted into bursts that make the four
+    // waves queue on the LDS pipe right after every barrier.
     // ---- part 1 ----------------------------------------------------------------------------------------------------------
-    if (DO_R) {
-#pragma unroll
-      for (int ks = 6; ks < 11; ++ks) at[ks] = tile_frag(i, ks);
-    }
     {
       f32x16 sacc;
 #pragma unroll
       for (int o = 0; o < 4; ++o) {
         if (DO_R) {
+          at[6 + o] = tile_frag(i, 6 + o);
+          if (o == 3) at[10] = tile_frag(i, 10);
 #pragma unroll
           for (int m = 3 * o; m < 3 * o + 3; ++m) {
             const int ks = m >> 1;
@@ -321,6 +324,13 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
             sacc = Elem<T>::mfma32(kop, qop[o], sacc);
           }
         }
+        if (DO_R && DO_PREV) {   // three reconstruction MFMAs dealt out among the rotation's VALU work, then the q-dot
+          XKV_SGB(0x8, 1); XKV_SGB(0x2, 7);
+          XKV_SGB(0x8, 1); XKV_SGB(0x2, 7);
+          XKV_SGB(0x8, 1); XKV_SGB(0x2, 10);
+          XKV_SGB(0x8, 1);
+        }
+        XKV_FENCE();
       }
       // lane (n32 = head, g2): register r of sacc = token 8 (r/4) + 4 g2 + r%4
       if (DO_PREV && n32 < G) {
@@ -333,32 +343,40 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     __syncthreads();        // B_b: partial scores of tile i-1 are visible
     // ---- part 2 ----------------------------------------------------------------------------------------------------------
     s16x4f tr[16];
+    const unsigned char* vt =
+        ring + ((i - 1) & (FRING - 1)) * FTILE + (8 * g4 + (n16 >> 2)) * FROW + (wave * 128 + 4 * (n16 & 3)) * 2;
+    auto tr_read = [&](int mb) {
+      tr[2 * mb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4f*)(vt + mb * 32));
+      tr[2 * mb + 1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4f*)(vt + mb * 32 + 4 * FROW));
+    };
+    auto recon_step = [&](int ks) {
+      k0 = Elem<T>::mfma32(breg[ks][0], at[ks], k0);
+      k1 = Elem<T>::mfma32(breg[ks][1], at[ks], k1);
+    };
+    if (DO_PREV) softmax_read();
     if (DO_R) {
-#pragma unroll
-      for (int ks = 11; ks < 16; ++ks) at[ks] = tile_frag(i, ks);
+      at[11] = tile_frag(i, 11);
+      recon_step(6);
     }
-    if (DO_PREV) {
-      const unsigned char* vt =
-          ring + ((i - 1) & (FRING - 1)) * FTILE + (8 * g4 + (n16 >> 2)) * FROW + (wave * 128 + 4 * (n16 & 3)) * 2;
-#pragma unroll
-      for (int mb = 0; mb < 8; ++mb) {
-        tr[2 * mb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4f*)(vt + mb * 32));
-        tr[2 * mb + 1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4f*)(vt + mb * 32 + 4 * FROW));
-      }
-    }
+    XKV_FENCE();
+    if (DO_PREV) { tr_read(0); tr_read(1); }
     if (DO_R) {
-      k0 = Elem<T>::mfma32(breg[6][0], at[6], k0);
-      k1 = Elem<T>::mfma32(breg[6][1], at[6], k1);
-      k0 = Elem<T>::mfma32(breg[7][0], at[7], k0);
-      k1 = Elem<T>::mfma32(breg[7][1], at[7], k1);
+      at[12] = tile_frag(i, 12);
+      at[13] = tile_frag(i, 13);
+      recon_step(7);
     }
-    if (DO_PREV) softmax_tile(i - 1);
+    XKV_FENCE();
+    if (DO_PREV) { softmax_tile(i - 1); tr_read(2); tr_read(3); }
     if (DO_R) {
-#pragma unroll
-      for (int ks = 8; ks < 11; ++ks) {
-        k0 = Elem<T>::mfma32(breg[ks][0], at[ks], k0);
-        k1 = Elem<T>::mfma32(breg[ks][1], at[ks], k1);
-      }
+      at[14] = tile_frag(i, 14);
+      recon_step(8);
+      recon_step(9);
+    }
+    XKV_FENCE();
+    if (DO_PREV) { tr_read(4); tr_read(5); tr_read(6); tr_read(7); }   // every transposed read of tile i-1 precedes B_c
+    if (DO_R) {
+      at[15] = tile_frag(i, 15);
+      recon_step(10);
       wait_vmcnt<8>();      // this wave's rows of tile i+1 have landed (the 8 loads of tile i+2 may be in flight)
     } else {
       wait_vmcnt<0>();
@@ -368,6 +386,12 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
                             // the transposed reads of tile i-1 have returned, so its ring slot is free
     // ---- part 3 ----------------------------------------------------------------------------------------------------------
     vec8 pb;
+    vec8 at_next[6], qop_next[4];
+    const T* qrow = qhat + (i & 1) * (8 * 128) + (n32 < G ? n32 : G - 1) * 128 + (dq * 2 + g2) * 8;
+    auto pv_step = [&](int mb) {
+      vec8 a = __builtin_bit_cast(vec8, (s16x8f)__builtin_shufflevector(tr[2 * mb], tr[2 * mb + 1], 0, 1, 2, 3, 4, 5, 6, 7));
+      acc[mb] = Elem<T>::mfma16(a, pb, acc[mb]);
+    };
     if (DO_PREV) {
       const float al = alpha_lds[n16];
       pb = ld16<vec8>(p_lds + n16 * FP_ROW + 8 * g4);
@@ -376,29 +400,28 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
         for (int mb = 0; mb < 8; ++mb) acc[mb] *= al;
       }
     }
-    vec8 at_next[6], qop_next[4];
     if (DO_R) {
-#pragma unroll
-      for (int ks = 0; ks < 6; ++ks) at_next[ks] = tile_frag(i + 1, ks);
-      const T* qrow = qhat + (i & 1) * (8 * 128) + (n32 < G ? n32 : G - 1) * 128 + (dq * 2 + g2) * 8;
-#pragma unroll
-      for (int o = 0; o < 4; ++o) qop_next[o] = ld16<vec8>(qrow + o * 32);
+      at_next[0] = tile_frag(i + 1, 0);
+      recon_step(11);
     }
+    XKV_FENCE();
 #pragma unroll
-    for (int u = 0; u < 5; ++u) {
-      if (DO_R) {
-        k0 = Elem<T>::mfma32(breg[11 + u][0], at[11 + u], k0);
-        k1 = Elem<T>::mfma32(breg[11 + u][1], at[11 + u], k1);
-        if (u == 0) issue_tile(i + 3, full_c);   // into the slot of tile i-1
-        if (u == 2) write_qhat(i + 1);           // buffer (i+1)&1 was last read in part 3 of iteration i-1
-      }
+    for (int u = 1; u < 5; ++u) {
       if (DO_PREV) {
-#pragma unroll
-        for (int mb = (u * 8) / 5; mb < ((u + 1) * 8) / 5; ++mb) {
-          vec8 a = __builtin_bit_cast(vec8, (s16x8f)__builtin_shufflevector(tr[2 * mb], tr[2 * mb + 1], 0, 1, 2, 3, 4, 5, 6, 7));
-          acc[mb] = Elem<T>::mfma16(a, pb, acc[mb]);
-        }
+        pv_step(2 * u - 2);
+        pv_step(2 * u - 1);
       }
+      if (DO_R) {
+        at_next[u] = tile_frag(i + 1, u);
+        if (u == 4) at_next[5] = tile_frag(i + 1, 5);
+        qop_next[u - 1] = ld16<vec8>(qrow + (u - 1) * 32);
+        recon_step(11 + u);
+        if (u == 1) issue_rows(i + 3, IC<0>(), IC<3>(), full_c);   // into the ring slot of tile i-1, whose readers are done
+        if (u == 2) issue_rows(i + 3, IC<3>(), IC<6>(), full_c);
+        if (u == 3) issue_rows(i + 3, IC<6>(), IC<8>(), full_c);
+        if (u == 4) write_qhat(i + 1);                             // buffer (i+1)&1 was last read in part 3 of iteration i-1
+      }
+      XKV_FENCE();
     }
     if (DO_R) {
 #pragma unroll
