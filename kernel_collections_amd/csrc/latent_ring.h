@@ -1,0 +1,25 @@
+// Parameters of the split-K stage 1 over dot-product scores, and the entry of its wide-row (LDS ring) variant.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace xkv {
+
+struct LatentParams {
+  const void* qn; const void* qn_lo; const void* qr;
+  const void* C; const void* R; const void* V;
+  int64_t sCb, sCl, sCh, sRb, sRl, sRh, sVb, sVl, sVh;   // element strides
+  int dn, dr, dv;
+  float* partial; float* lse; void* scores; int scores_dtype;
+  const int32_t* num_splits; const int32_t* kv_lens;
+  int hq, groups, kv_len, max_splits, total_wg;
+  float sm_scale, logit_cap;
+};
+typedef LatentParams RingParams;
+
+// True when the shape is one the ring kernel is built for (512-wide latent rows, optionally + 64 RoPE features, V the
+// latent itself or scores-only); everything else runs the register-staged kernel.
+bool ring_eligible(const RingParams& p, bool vshared);
+int launch_ring(const RingParams& p, int batch, int dtype, hipStream_t st);
+
+}  // namespace xkv

@@ -14,19 +14,9 @@
 // When V is the same tensor as C (MLA latent, xKV with a basis shared by K and V) the tile is
 // loaded once and used for both products.
 #include "xkv_common.h"
+#include "latent_ring.h"
 
 namespace xkv {
-
-struct LatentParams {
-  const void* qn; const void* qn_lo; const void* qr;
-  const void* C; const void* R; const void* V;
-  int64_t sCb, sCl, sCh, sRb, sRl, sRh, sVb, sVl, sVh;
-  int dn, dr, dv;
-  float* partial; float* lse; void* scores; int scores_dtype;
-  const int32_t* num_splits; const int32_t* kv_lens;
-  int hq, groups, kv_len, max_splits, total_wg;
-  float sm_scale, logit_cap;
-};
 
 // Workgroups are dealt round-robin over the 8 XCDs by linear id.  Remap so that logically
 // consecutive workgroups (which share kv-group tiles) sit on the same XCD, hence the same L2.
@@ -413,6 +403,7 @@ extern "C" int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_oper
   const bool vshared = !scores_only && V.ptr == C.ptr && V.stride_b == C.stride_b && V.stride_l == C.stride_l &&
                        V.stride_h == C.stride_h && V.dim == C.dim;
   hipStream_t st = (hipStream_t)stream;
+  if (ring_eligible(p, vshared)) return launch_ring(p, batch, dtype, st);
   if (dtype == XKV_BF16)
     return hg <= 16 ? dispatch_latent<__bf16, 1>(p, batch, vshared, st) : dispatch_latent<__bf16, 2>(p, batch, vshared, st);
   return hg <= 16 ? dispatch_latent<_Float16, 1>(p, batch, vshared, st) : dispatch_latent<_Float16, 2>(p, batch, vshared, st);

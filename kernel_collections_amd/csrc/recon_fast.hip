@@ -80,21 +80,6 @@ __global__ __launch_bounds__(256) void pack_b_kernel(const T* __restrict__ kB, T
   }
 }
 
-// max / sum over each row of 16 lanes, result in every lane of the row (DPP butterflies, no LDS traffic)
-template <bool IS_MAX> __device__ __forceinline__ float row16_reduce(float x) {
-#define XKV_DPP_STEP(ctrl)                                                                                       \
-  {                                                                                                              \
-    const float y = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), ctrl, 0xf, 0xf, false)); \
-    x = IS_MAX ? fmaxf(x, y) : x + y;                                                                            \
-  }
-  XKV_DPP_STEP(0xB1)   // quad_perm [1,0,3,2]
-  XKV_DPP_STEP(0x4E)   // quad_perm [2,3,0,1]
-  XKV_DPP_STEP(0x141)  // row_half_mirror
-  XKV_DPP_STEP(0x140)  // row_mirror
-#undef XKV_DPP_STEP
-  return x;
-}
-
 template <int V> using IC = std::integral_constant<int, V>;
 #define XKV_FENCE() __builtin_amdgcn_sched_barrier(0)
 #define XKV_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)   // 0x8 MFMA, 0x2 VALU, 0x100 LDS read, 0x200 LDS write
@@ -243,12 +228,12 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     s0 = tok < end ? s0 * p.sm_scale : NEG_INF;
     s1 = tok + 1 < end ? s1 * p.sm_scale : NEG_INF;
     // the reference maximum only moves when the tile maximum exceeds it by LAZY_RESCALE (branch-free: alpha = 1 otherwise)
-    const float mx = row16_reduce<true>(fmaxf(s0, s1));
+    const float mx = row_reduce<true, 16>(fmaxf(s0, s1));
     const float m_new = mx > m_ref + LAZY_RESCALE ? mx : m_ref;
     const float alpha = __expf(m_ref - m_new);
     m_ref = m_new;
     const float e0 = __expf(s0 - m_ref), e1 = __expf(s1 - m_ref);
-    l_run = l_run * alpha + row16_reduce<false>(e0 + e1);
+    l_run = l_run * alpha + row_reduce<false, 16>(e0 + e1);
     T* pd = p_lds + sm_head * FP_ROW + 2 * n16;
     pd[0] = from_f32<T>(sm_valid ? e0 : 0.f);
     pd[1] = from_f32<T>(sm_valid ? e1 : 0.f);

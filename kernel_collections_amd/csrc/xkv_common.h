@@ -79,6 +79,23 @@ __device__ __forceinline__ float group4_sum(float v) {
   return v;
 }
 
+// max / sum over each aligned group of WIDTH (8 or 16) consecutive lanes, result in every lane of the group
+// (DPP butterflies inside a 16-lane row: no LDS traffic, unlike __shfl_xor)
+template <bool IS_MAX, int WIDTH> __device__ __forceinline__ float row_reduce(float x) {
+  static_assert(WIDTH == 8 || WIDTH == 16, "row_reduce width");
+#define XKV_DPP_STEP(ctrl)                                                                                       \
+  {                                                                                                              \
+    const float y = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), ctrl, 0xf, 0xf, false)); \
+    x = IS_MAX ? fmaxf(x, y) : x + y;                                                                            \
+  }
+  XKV_DPP_STEP(0xB1)   // quad_perm [1,0,3,2]
+  XKV_DPP_STEP(0x4E)   // quad_perm [2,3,0,1]
+  XKV_DPP_STEP(0x141)  // row_half_mirror
+  if (WIDTH == 16) XKV_DPP_STEP(0x140)  // row_mirror
+#undef XKV_DPP_STEP
+  return x;
+}
+
 inline int launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? XKV_OK : (int)e;
