@@ -178,7 +178,7 @@ def bench_c2(args, dev):
     q3 = q.reshape(B, Hq, d)
     hi, lo = ops.absorb_q(q3, Bm)
     out = torch.empty((B, Hq, 1, L), dtype=torch.float32, device=dev)
-    S = args.splits or ops.occupancy_splits(B, 1, L)
+    S = args.splits or ops.latent_splits(B, 1, L, r)
     ns = ops.uniform_splits(B, S, dev)
 
     def scan(i):
@@ -193,7 +193,7 @@ def bench_c2(args, dev):
         "metric": "us_per_qAB_no_pe_call", "value": round(us, 2), "unit": "us", "higher_is_better": False,
         "ms_per_step": total_ms / args.steps,
         "config": {"workload": "c2 qAB_no_pe scores: batch 8, 32q/8kv, d128, L16384, rank 512, bf16 in / fp32 out", "kv_splits": S},
-        "roofline": {"bound": "hbm", "kernel": "latent_stage1_kernel(scores)", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+        "roofline": {"bound": "hbm", "kernel": "latent_ring_kernel(scores)", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None,
                      "kernel_avg_us": round(k_avg_ms * 1e3, 2), "kernel_median_us": round(k_med_ms * 1e3, 2),
                      "algorithmic_bytes": algo_bytes},
@@ -211,7 +211,7 @@ def bench_c5(args, dev):
     scale = 1 / math.sqrt(192)
     total_ms = time_loop(lambda i: mla2.mla_decode_attention_fwd(qn, qr, ckv, kpe, scale), args.steps, args.warmup)
     us = total_ms * 1e3 / args.steps
-    S = args.splits or ops.occupancy_splits(B, 1, L)
+    S = args.splits or ops.latent_splits(B, 1, L, 512)
     ns = ops.uniform_splits(B, S, dev)
     partial, lse = ops.workspaces(B, H, S, c, dev)
     k_avg_ms, k_med_ms = time_kernel(lambda i: mla2.decoding_stage1(qn, qr, ckv, kpe, partial, lse, ns, S, scale),
@@ -223,7 +223,7 @@ def bench_c5(args, dev):
         "metric": "us_per_mla_decode_step", "value": round(us, 2), "unit": "us", "higher_is_better": False,
         "ms_per_step": total_ms / args.steps,
         "config": {"workload": "c5 MLA absorbed decode: batch 64, 16 heads, latent 512 + rope 64, ctx 8192, bf16", "kv_splits": S},
-        "roofline": {"bound": "hbm", "kernel": "latent_stage1_kernel", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+        "roofline": {"bound": "hbm", "kernel": "latent_ring_kernel", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None,
                      "kernel_avg_us": round(k_avg_ms * 1e3, 2), "kernel_median_us": round(k_med_ms * 1e3, 2),
                      "algorithmic_bytes": algo_bytes, "mfma_TFLOPs": round(flops / (k_avg_ms * 1e-3) / 1e12, 1)},
@@ -243,6 +243,10 @@ def bench_c4(args, dev, vfact):
     K = randn_dev((B, Lmax, Hkv, d), 1.0, dev, gen=gen)
     q = randn_dev((B, Hq, d), 1.0, dev, gen=gen)
     o = torch.empty_like(q)
+    if vfact:
+        split = args.splits or 1024   # one workgroup serves all 32 heads of a split, so the splits are shorter than plain GQA's
+    elif args.splits:
+        split = args.splits
     ns_l = [-(-n // split) for n in lens]
     S = max(ns_l)
     ns = torch.tensor(ns_l, dtype=torch.int32, device=dev)
@@ -264,10 +268,11 @@ def bench_c4(args, dev, vfact):
     return {
         "metric": "us_per_ragged_decode_step", "value": round(us, 2), "unit": "us", "higher_is_better": False,
         "ms_per_step": total_ms / args.steps,
-        "config": {"workload": "c4 ragged split-K GQA%s: batch 32, lens log-uniform [1024,131072], split 4096"
-                               % (" V-factorised r512" if vfact else ""), "sum_len": sum(lens), "max_len": Lmax,
+        "config": {"workload": "c4 ragged split-K GQA%s: batch 32, lens log-uniform [1024,131072], split %d"
+                               % (" V-factorised r512" if vfact else "", split), "sum_len": sum(lens), "max_len": Lmax,
                    "kv_splits_max": S},
-        "roofline": {"bound": "hbm", "kernel": "latent_stage1_kernel", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+        "roofline": {"bound": "hbm", "kernel": "latent_ring_kernel" if vfact else "latent_stage1_kernel",
+                     "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None,
                      "note": "whole call (stage 1 + merge) over algorithmic bytes", "algorithmic_bytes": algo_bytes},
         "cpu_baseline": None,

@@ -62,6 +62,14 @@ int xkv_absorb_q(const void* q, const void* B, void* qt_hi, void* qt_lo,
                  int64_t stride_B_b, int64_t stride_B_h, int64_t stride_B_r,
                  int dtype, void* stream);
 
+/* Block-diagonal query: out[b, h, kh * d + c] = q[b, h, c] when kh == h / (hq / hkv), else 0; q is [batch, hq, d],
+ * out [batch, hq, hkv * d], both contiguous.  Against it the per-head keys of a token, stored side by side
+ * ([batch, kv_len, hkv, d] with unit head stride d), behave as one hkv*d-wide row shared by every head, so
+ * xkv_latent_stage1 can serve all heads of a sequence from one workgroup (n_kv_groups = 1) and read a value basis
+ * that the heads share once per token instead of once per kv head.  No reference counterpart: the reference has the
+ * V-only factorised decode only in eager form (attention.py:202-274).   d % 8 == 0. */
+int xkv_blockdiag_q(const void* q, void* out, int batch, int hq, int hkv, int d, int dtype, void* stream);
+
 /* Operand descriptors of the generic split-K stage 1. */
 typedef struct {
   const void* ptr;     /* [batch, kv_len, heads?, dim]; NULL = absent                      */

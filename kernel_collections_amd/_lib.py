@@ -16,7 +16,7 @@ ABI_VERSION = 1
 
 EXPORTS = (
     "xkv_abi_version", "xkv_error_string", "xkv_rope_table", "xkv_absorb_q",
-    "xkv_latent_stage1", "xkv_recon_stage1", "xkv_recon_workspace_bytes", "xkv_merge_stage2",
+    "xkv_blockdiag_q", "xkv_latent_stage1", "xkv_recon_stage1", "xkv_recon_workspace_bytes", "xkv_merge_stage2",
 )
 
 
@@ -42,6 +42,8 @@ def _declare(lib):
     lib.xkv_absorb_q.restype = c_int
     lib.xkv_absorb_q.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                  c_int64, c_int64, c_int64, c_int, c_void_p]
+    lib.xkv_blockdiag_q.restype = c_int
+    lib.xkv_blockdiag_q.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]
     lib.xkv_latent_stage1.restype = c_int
     lib.xkv_latent_stage1.argtypes = [QOperand, c_void_p, QOperand, KVOperand, KVOperand, KVOperand,
                                       c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,

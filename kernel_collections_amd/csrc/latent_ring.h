@@ -18,8 +18,9 @@ struct LatentParams {
 typedef LatentParams RingParams;
 
 // True when the shape is one the ring kernel is built for (512-wide latent rows, optionally + 64 RoPE features, V the
-// latent itself or scores-only); everything else runs the register-staged kernel.
+// latent itself or scores-only; or two row streams: keys 512 / 1024 wide, values 512 wide); everything else runs the
+// register-staged kernel.
 bool ring_eligible(const RingParams& p, bool vshared);
-int launch_ring(const RingParams& p, int batch, int dtype, hipStream_t st);
+int launch_ring(const RingParams& p, int batch, bool vshared, int dtype, hipStream_t st);
 
 }  // namespace xkv

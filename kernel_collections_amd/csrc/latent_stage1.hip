@@ -403,7 +403,7 @@ extern "C" int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_oper
   const bool vshared = !scores_only && V.ptr == C.ptr && V.stride_b == C.stride_b && V.stride_l == C.stride_l &&
                        V.stride_h == C.stride_h && V.dim == C.dim;
   hipStream_t st = (hipStream_t)stream;
-  if (ring_eligible(p, vshared)) return launch_ring(p, batch, dtype, st);
+  if (ring_eligible(p, vshared)) return launch_ring(p, batch, vshared, dtype, st);
   if (dtype == XKV_BF16)
     return hg <= 16 ? dispatch_latent<__bf16, 1>(p, batch, vshared, st) : dispatch_latent<__bf16, 2>(p, batch, vshared, st);
   return hg <= 16 ? dispatch_latent<_Float16, 1>(p, batch, vshared, st) : dispatch_latent<_Float16, 2>(p, batch, vshared, st);

@@ -38,7 +38,7 @@ __global__ __launch_bounds__(256) void absorb_q_kernel(
   for (int i = threadIdx.x; i < G * d; i += blockDim.x) qs[i] = to_f32(qb[i]);
   __syncthreads();
   const T* Bh = B + b * sBb + kh * sBh;
-  for (int rho = threadIdx.x; rho < rank; rho += blockDim.x) {
+  for (int rho = blockIdx.z * blockDim.x + threadIdx.x; rho < rank; rho += blockDim.x * gridDim.z) {
     const T* row = Bh + rho * sBr;
     for (int g0 = 0; g0 < G; g0 += 4) {
       float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -62,6 +62,68 @@ __global__ __launch_bounds__(256) void absorb_q_kernel(
         }
     }
   }
+}
+
+// Same product for head_dim 64 / 128 with coalesced reads: TPR = d / 8 consecutive lanes cover one row of B (16 bytes
+// each), 256 / TPR rows per pass, 64 rows per workgroup; the per-row dot products are finished by a DPP reduction.
+template <typename T, int TPR>
+__global__ __launch_bounds__(256) void absorb_q_rows_kernel(
+    const T* __restrict__ q, const T* __restrict__ B, T* __restrict__ qt_hi, T* __restrict__ qt_lo,
+    int hq, int hkv, int rank, int64_t sBb, int64_t sBh, int64_t sBr) {
+  typedef typename Elem<T>::vec8 vec8;
+  constexpr int D = TPR * 8, RPP = 256 / TPR;
+  __shared__ float qs[32 * D];
+  const int kh = blockIdx.x, b = blockIdx.y, G = hq / hkv;
+  const T* qb = q + ((int64_t)b * hq + (int64_t)kh * G) * D;
+  for (int i = threadIdx.x; i < G * D; i += 256) qs[i] = to_f32(qb[i]);
+  __syncthreads();
+  const int sub = threadIdx.x % TPR, rr = threadIdx.x / TPR;
+  const T* Bh = B + b * sBb + kh * sBh;
+  for (int r0 = 0; r0 < 64; r0 += RPP) {
+    const int rho = blockIdx.z * 64 + r0 + rr;
+    const bool live = rho < rank;
+    float x[8];
+    {
+      vec8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (live) v = ld16<vec8>(Bh + (int64_t)rho * sBr + sub * 8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = to_f32(v[e]);
+    }
+    for (int g = 0; g < G; ++g) {
+      const f32x4 qa = *reinterpret_cast<const f32x4*>(qs + g * D + sub * 8);
+      const f32x4 qb4 = *reinterpret_cast<const f32x4*>(qs + g * D + sub * 8 + 4);
+      float a = x[0] * qa[0] + x[1] * qa[1] + x[2] * qa[2] + x[3] * qa[3] + x[4] * qb4[0] + x[5] * qb4[1] + x[6] * qb4[2] +
+                x[7] * qb4[3];
+      a = row_reduce<false, TPR>(a);
+      if (live && sub == (g % TPR)) {
+        const int64_t o = ((int64_t)b * hq + (int64_t)kh * G + g) * rank + rho;
+        const T hi = from_f32<T>(a);
+        qt_hi[o] = hi;
+        if (qt_lo) qt_lo[o] = from_f32<T>(a - to_f32(hi));
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------------------------
+// Block-diagonal query: out[b, h, kh * d + c] = q[b, h, c] if kh == h / G else 0.  With it the per-head keys of a token,
+// stored side by side ([batch, kv_len, hkv * d]), act as ONE wide row shared by every head, so a single workgroup can
+// serve all query heads of a sequence (and read a value basis shared by the heads once instead of once per kv head).
+// ----------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void blockdiag_q_kernel(const T* __restrict__ q, T* __restrict__ out, int hq, int hkv, int d,
+                                                          int64_t total8) {
+  typedef typename Elem<T>::vec8 vec8;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;   // one 8-element packet of out
+  if (i >= total8) return;
+  const int ppr = hkv * d / 8, dp = d / 8;
+  const int64_t row = i / ppr;            // b * hq + h
+  const int pk = (int)(i - row * ppr);
+  const int kh = pk / dp, c = (pk - kh * dp) * 8;
+  const int h = (int)(row % hq), G = hq / hkv;
+  vec8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (kh == h / G) v = ld16<vec8>(q + row * d + c);
+  st16(out + i * 8, v);
 }
 
 // ----------------------------------------------------------------------------------------------
@@ -221,15 +283,33 @@ extern "C" int xkv_absorb_q(const void* q, const void* B, void* qt_hi, void* qt_
   if (hq % hkv || hq / hkv > 32 || d > 256 || d % 8) return XKV_EUNSUPPORTED;
   if (sBr % 8 || sBh % 8 || sBb % 8 || ((uintptr_t)B & 15)) return XKV_EALIGN;
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid(hkv, batch), block(256);
-  if (dtype == XKV_BF16)
-    absorb_q_kernel<__bf16><<<grid, block, 0, st>>>((const __bf16*)q, (const __bf16*)B, (__bf16*)qt_hi, (__bf16*)qt_lo,
-                                                    hq, hkv, d, rank, sBb, sBh, sBr);
-  else if (dtype == XKV_F16)
-    absorb_q_kernel<_Float16><<<grid, block, 0, st>>>((const _Float16*)q, (const _Float16*)B, (_Float16*)qt_hi,
-                                                      (_Float16*)qt_lo, hq, hkv, d, rank, sBb, sBh, sBr);
-  else
-    return XKV_EDTYPE;
+  if (dtype != XKV_BF16 && dtype != XKV_F16) return XKV_EDTYPE;
+  const dim3 block(256);
+#define XKV_ABSORB(T)                                                                                                         \
+  if (d == 128)                                                                                                               \
+    absorb_q_rows_kernel<T, 16><<<dim3(hkv, batch, (rank + 63) / 64), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,    \
+                                                                                        (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr); \
+  else if (d == 64)                                                                                                           \
+    absorb_q_rows_kernel<T, 8><<<dim3(hkv, batch, (rank + 63) / 64), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,     \
+                                                                                       (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr); \
+  else                                                                                                                        \
+    absorb_q_kernel<T><<<dim3(hkv, batch, (rank + 255) / 256), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi, (T*)qt_lo, \
+                                                                                 hq, hkv, d, rank, sBb, sBh, sBr);
+  if (dtype == XKV_BF16) { XKV_ABSORB(__bf16) } else { XKV_ABSORB(_Float16) }
+#undef XKV_ABSORB
+  return launch_status();
+}
+
+extern "C" int xkv_blockdiag_q(const void* q, void* out, int batch, int hq, int hkv, int d, int dtype, void* stream) {
+  if (!q || !out || batch <= 0 || hq <= 0 || hkv <= 0 || d <= 0) return XKV_EINVAL;
+  if (hq % hkv || d % 8) return XKV_EUNSUPPORTED;
+  if (((uintptr_t)q & 15) || ((uintptr_t)out & 15)) return XKV_EALIGN;
+  const int64_t total8 = (int64_t)batch * hq * hkv * d / 8;
+  const dim3 grid((unsigned)((total8 + 255) / 256)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == XKV_BF16) blockdiag_q_kernel<__bf16><<<grid, block, 0, st>>>((const __bf16*)q, (__bf16*)out, hq, hkv, d, total8);
+  else if (dtype == XKV_F16) blockdiag_q_kernel<_Float16><<<grid, block, 0, st>>>((const _Float16*)q, (_Float16*)out, hq, hkv, d, total8);
+  else return XKV_EDTYPE;
   return launch_status();
 }
 

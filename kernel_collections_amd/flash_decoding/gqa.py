@@ -58,8 +58,17 @@ def decode_attention_fwd_v_factorized(q, k_buffer, v_A_buffer, v_B_buffer, o, nu
     q3 = ops._q3(q)
     k_buffer, v_A_buffer = ops.as_rows(k_buffer), ops.as_rows(v_A_buffer)
     partial, lse = ops.workspaces(batch, hq, S, rv, q.device)
-    ops.latent_stage1(q3, None, None,
-                      (k_buffer, k_buffer.stride(0), k_buffer.stride(1), k_buffer.stride(2), d), None,
-                      (v_A_buffer, v_A_buffer.stride(0), v_A_buffer.stride(1), 0, rv),
-                      partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale))
+    if hkv * d in (512, 1024) and rv == 512 and hq <= 32 and k_buffer.stride(2) == d:
+        # all heads from one workgroup: the token's keys are one hkv*d-wide row against a block-diagonal query, and the
+        # value basis (shared by the heads) is read once per token instead of once per kv head
+        qbd = ops.blockdiag_q(q3, hkv)
+        ops.latent_stage1(qbd, None, None,
+                          (k_buffer, k_buffer.stride(0), k_buffer.stride(1), 0, hkv * d), None,
+                          (v_A_buffer, v_A_buffer.stride(0), v_A_buffer.stride(1), 0, rv),
+                          partial, lse, None, splits, lens, batch, hq, 1, kv_len, S, float(sm_scale))
+    else:
+        ops.latent_stage1(q3, None, None,
+                          (k_buffer, k_buffer.stride(0), k_buffer.stride(1), k_buffer.stride(2), d), None,
+                          (v_A_buffer, v_A_buffer.stride(0), v_A_buffer.stride(1), 0, rv),
+                          partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale))
     return ops.merge_stage2(partial, lse, o, v_B_buffer, splits, lens, batch, hq, hkv, kv_len, S)

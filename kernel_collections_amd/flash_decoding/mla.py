@@ -42,7 +42,7 @@ def decode_attention_fwd(q, k_buffer, v_buffer, o, sm_scale=1.0, logit_cap=0.0):
     groups = num_kv_heads * per_kv_groups
     sh = k_buffer.stride(2) if per_kv_groups == 1 else 0
     svh = v_buffer.stride(2) if per_kv_groups == 1 else 0
-    S = ops.occupancy_splits(batch, groups, kv_len)
+    S = ops.latent_splits(batch, groups, kv_len, dn)
     splits = ops.uniform_splits(batch, S, q.device)
     partial, lse = ops.workspaces(batch, num_q_heads, S, dv, q.device)
     C = (k_buffer, k_buffer.stride(0), k_buffer.stride(1), sh, dn)

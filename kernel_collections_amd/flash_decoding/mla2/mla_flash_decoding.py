@@ -17,7 +17,7 @@ def _run(q_nope, q_rope, kv_nope, k_rope, sm_scale):
     batch, num_q_heads, width = q_nope.shape
     kv_len = kv_nope.shape[1]
     groups = ops.head_groups(num_q_heads)
-    S = ops.occupancy_splits(batch, groups, kv_len)
+    S = ops.latent_splits(batch, groups, kv_len, width)
     splits = ops.uniform_splits(batch, S, q_nope.device)
     attn_logits, attn_lse = ops.workspaces(batch, num_q_heads, S, width, q_nope.device)
     decoding_stage1(q_nope, q_rope, kv_nope, k_rope, attn_logits, attn_lse, splits, S, sm_scale)

@@ -60,6 +60,14 @@ def occupancy_splits(batch: int, groups: int, kv_len: int, tile: int = 64, waves
     return max(1, min(want, cap))
 
 
+def latent_splits(batch: int, groups: int, kv_len: int, width: int) -> int:
+    """Split count for the dot-product stage 1: 512-wide rows run the LDS-ring kernel (one workgroup per CU,
+    32-token tiles), everything else the register-staged one (two workgroups per CU, 64-token tiles)."""
+    if width == 512:
+        return occupancy_splits(batch, groups, kv_len, tile=32, waves=1)
+    return occupancy_splits(batch, groups, kv_len)
+
+
 def _row_ok(t: torch.Tensor) -> bool:
     """Unit stride on the feature axis, every other stride a multiple of 8 elements, 16-byte base."""
     if t.stride(-1) != 1 or t.data_ptr() % 16:
@@ -100,6 +108,15 @@ def absorb_q(q3: torch.Tensor, Bk: torch.Tensor, want_lo: bool = True) -> Tuple[
                                   c_int64(Bk.stride(0)), c_int64(Bk.stride(1)), c_int64(Bk.stride(2)),
                                   dtype_code(q3.dtype), stream_ptr(q3)), "xkv_absorb_q")
     return hi, lo
+
+
+def blockdiag_q(q3: torch.Tensor, hkv: int) -> torch.Tensor:
+    """``[batch, hq, d]`` -> ``[batch, hq, hkv * d]`` with head h's row non-zero only in the slot of its kv head."""
+    batch, hq, d = q3.shape
+    out = torch.empty((batch, hq, hkv * d), dtype=q3.dtype, device=q3.device)
+    check(_lib.lib().xkv_blockdiag_q(ptr(q3), ptr(out), batch, hq, hkv, d, dtype_code(q3.dtype), stream_ptr(q3)),
+          "xkv_blockdiag_q")
+    return out
 
 
 def latent_stage1(qn, qn_lo, qr, C, R, V, partial, lse, scores, num_kv_splits, kv_lens,

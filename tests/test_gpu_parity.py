@@ -237,6 +237,32 @@ def test_gqa_ragged_plain_and_v_factorized(dev):
     check_out(o2, ref_v, "ragged V-factorised")
 
 
+@pytest.mark.parametrize("dtype", [BF, FP])
+@pytest.mark.parametrize("b,hq,hkv,L,rv,S", [(2, 32, 8, 1500, 512, 4),    # all heads from one workgroup (block-diagonal query)
+                                             (1, 16, 4, 333, 512, 2),     # same, 512-wide key rows
+                                             (2, 8, 2, 700, 256, 3)])     # one workgroup per kv head
+def test_gqa_v_factorized(dev, dtype, b, hq, hkv, L, rv, S):
+    d = 128
+    q, K = gen((b, hq, d), dtype=dtype, seed=1), gen((b, L, hkv, d), dtype=dtype, seed=2)
+    vA, vB = gen((b, L, rv), dtype=dtype, seed=3), gen((b, hkv, rv, d), std=rv ** -0.5, dtype=dtype, seed=4)
+    scale = d ** -0.5
+    ref = oracle.gqa_v_only(*f32(q.unsqueeze(2), K.transpose(1, 2), vA, vB), sm_scale=scale)[:, :, 0]
+    qd, Kd, vAd, vBd = dev_(dev, q, K, vA, vB)
+    o = torch.zeros_like(qd)
+    gqa.decode_attention_fwd_v_factorized(qd, Kd, vAd, vBd, o, splits_t([S] * b, dev), S, scale)
+    check_out(o, ref, "V-factorised")
+
+
+def test_blockdiag_q_is_exact(dev):
+    b, hq, hkv, d = 3, 32, 8, 128
+    q = gen((b, hq, d), dtype=BF, seed=7).to(dev)
+    out = ops.blockdiag_q(q, hkv).view(b, hq, hkv, d)
+    ref = torch.zeros_like(out)
+    for h in range(hq):
+        ref[:, h, h // (hq // hkv)] = q[:, h]
+    assert torch.equal(out, ref)
+
+
 # ------------------------------------------------------------------------------------ MLA
 @pytest.mark.parametrize("dtype", [BF, FP])
 def test_mla2(dev, dtype):
