@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256) void latent_ring_kernel(const RingParams p) {
   const int n16 = lane & 15, g4 = lane >> 4;
   const int tb = wave % NTB, kh = wave / NTB;
 
-  int wg = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);   // XCD-aware: neighbours in (group, split) share an L2
+  const int wg = xcd_cluster_remap(blockIdx.x, p.groups);   // the kv groups of one (sequence, split) share an L2
   if (wg >= p.total_wg) return;
   const int group = wg % p.groups;
   const int split = (wg / p.groups) % p.max_splits;
@@ -361,7 +361,7 @@ static int launch_ring_t(const RingParams& p, int batch, hipStream_t st) {
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SHM);
   if (e != hipSuccess) return (int)e;
   const int total = batch * p.groups * p.max_splits;
-  kern<<<dim3((total + 7) & ~7), dim3(256), SHM, st>>>(p);
+  kern<<<dim3(xcd_grid(total, p.groups)), dim3(256), SHM, st>>>(p);
   return launch_status();
 }
 

@@ -18,12 +18,6 @@
 
 namespace xkv {
 
-// Workgroups are dealt round-robin over the 8 XCDs by linear id.  Remap so that logically
-// consecutive workgroups (which share kv-group tiles) sit on the same XCD, hence the same L2.
-__device__ __forceinline__ int xcd_remap(int id, int total /* multiple of 8 */) {
-  return (id & 7) * (total >> 3) + (id >> 3);
-}
-
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 
@@ -53,7 +47,7 @@ __global__ __launch_bounds__(256) void latent_stage1_kernel(const LatentParams p
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n16 = lane & 15, g4 = lane >> 4;
 
-  int wg = xcd_remap(blockIdx.x, gridDim.x);
+  const int wg = xcd_cluster_remap(blockIdx.x, p.groups);   // the kv groups of one (sequence, split) share an L2
   if (wg >= p.total_wg) return;
   const int group = wg % p.groups;
   const int split = (wg / p.groups) % p.max_splits;
@@ -339,7 +333,7 @@ static int launch_latent(const LatentParams& p, int batch, hipStream_t st) {
                                      (int)shm);
   if (e != hipSuccess) return (int)e;
   const int total = batch * p.groups * p.max_splits;
-  const int grid = (total + 7) & ~7;
+  const int grid = xcd_grid(total, p.groups);
   kern<<<dim3(grid), dim3(256), shm, st>>>(p);
   return launch_status();
 }

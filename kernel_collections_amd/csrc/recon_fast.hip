@@ -94,8 +94,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   const int n32 = lane & 31, g2 = lane >> 5;
   const int n16 = lane & 15, g4 = lane >> 4;
 
-  const int total8 = gridDim.x;
-  int wg = (blockIdx.x & 7) * (total8 >> 3) + (blockIdx.x >> 3);   // XCD-aware: the 8 kv heads of a tile stream share an L2
+  const int wg = xcd_cluster_remap(blockIdx.x, p.hkv);   // the kv heads of one (sequence, split) stream the same rows: one L2
   if (wg >= p.total_wg) return;
   const int kh = wg % p.hkv;
   const int split = (wg / p.hkv) % p.max_splits;
@@ -467,7 +466,7 @@ int launch_recon_fast_t(const FastParams& p, const void* kB, int64_t sBb, int64_
                                      (int)FAST_SHM);
   if (e != hipSuccess) return (int)e;
   const int total = batch * p.hkv * p.max_splits;
-  kern<<<dim3((total + 7) & ~7), dim3(256), FAST_SHM, st>>>(p);
+  kern<<<dim3(xcd_grid(total, p.hkv)), dim3(256), FAST_SHM, st>>>(p);
   return launch_status();
 }
 

@@ -33,7 +33,6 @@ struct ReconParams {
   const void* sin_cos; int64_t sSCl;
 };
 
-__device__ __forceinline__ int xcd_remap_r(int id, int total) { return (id & 7) * (total >> 3) + (id >> 3); }
 
 typedef short s16x4r __attribute__((ext_vector_type(4)));
 typedef short s16x8r __attribute__((ext_vector_type(8)));
@@ -59,7 +58,7 @@ __global__ __launch_bounds__(256) void recon_stage1_kernel(const ReconParams p) 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n16 = lane & 15, g4 = lane >> 4;
 
-  int wg = xcd_remap_r(blockIdx.x, gridDim.x);
+  const int wg = xcd_cluster_remap(blockIdx.x, p.hkv);   // the kv heads of one (sequence, split) share an L2
   if (wg >= p.total_wg) return;
   const int kh = wg % p.hkv;
   const int split = (wg / p.hkv) % p.max_splits;
@@ -333,7 +332,7 @@ static int launch_recon(const ReconParams& p, int batch, hipStream_t st) {
                                      (int)shm);
   if (e != hipSuccess) return (int)e;
   const int total = batch * p.hkv * p.max_splits;
-  kern<<<dim3((total + 7) & ~7), dim3(256), shm, st>>>(p);
+  kern<<<dim3(xcd_grid(total, p.hkv)), dim3(256), shm, st>>>(p);
   return launch_status();
 }
 

@@ -137,36 +137,56 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     const TB* __restrict__ vB, int64_t sVb, int64_t sVh, int64_t sVr, int d_out,
     const int32_t* __restrict__ num_kv_splits, const int32_t* __restrict__ kv_lens,
     int hq, int hkv, int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh) {
-  extern __shared__ float merged[];  // [G][dv]
+  extern __shared__ float merged[];  // [G][dv], then the split weights [G][max_splits]
   __shared__ float fin[4 * 256];     // per-head-block totals of the up-projection
   const int kh = blockIdx.x, b = blockIdx.y, G = hq / hkv;
   const int L = kv_lens ? kv_lens[b] : kv_len;
   const int ns = num_kv_splits[b];
+  float* wts = merged + G * dv;
+  // weights of the live splits, w_i = exp(lse_i - max lse) / sum: one wave per head, lanes stride over the splits
+  {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int gi = wave; gi < G; gi += 4) {
+      const float* pl = lse + ((int64_t)b * hq + kh * G + gi) * max_splits;
+      float mx = NEG_INF;
+      for (int i = lane; i < max_splits; i += 64) {
+        int s0, e0;
+        split_bounds(L, ns, i, s0, e0);
+        const float v = e0 > s0 ? pl[i] : NEG_INF;   // dead splits were never written
+        wts[gi * max_splits + i] = v;
+        mx = fmaxf(mx, v);
+      }
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+      float sum = 0.f;
+      for (int i = lane; i < max_splits; i += 64) {
+        const float v = wts[gi * max_splits + i];
+        const float w = v == NEG_INF ? 0.f : __expf(v - mx);
+        wts[gi * max_splits + i] = w;
+        sum += w;
+      }
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) sum += __shfl_xor(sum, o);
+      const float inv = 1.f / sum;
+      for (int i = lane; i < max_splits; i += 64) wts[gi * max_splits + i] *= inv;
+    }
+  }
+  __syncthreads();
   for (int idx = threadIdx.x; idx < G * dv; idx += blockDim.x) {
     const int gi = idx / dv, c = idx - gi * dv;
     const int h = kh * G + gi;
-    const float* pl = lse + ((int64_t)b * hq + h) * max_splits;
     const float* pp = partial + ((int64_t)b * hq + h) * max_splits * (int64_t)dv + c;
-    float g_lse = NEG_INF, g_sum = 0.f, acc = 0.f;
+    const float* w = wts + gi * max_splits;
+    float acc = 0.f;
+#pragma unroll 8
     for (int i = 0; i < max_splits; ++i) {
-      int s, e;
-      split_bounds(L, ns, i, s, e);
-      if (e > s) {
-        float tv = pp[(int64_t)i * dv];
-        float in = pl[i];
-        float nl = fmaxf(in, g_lse);
-        float old_scale = __expf(g_lse - nl);
-        float w = __expf(in - nl);
-        acc = acc * old_scale + w * tv;
-        g_sum = g_sum * old_scale + w;
-        g_lse = nl;
-      }
+      const float wi = w[i];
+      if (wi != 0.f) acc += wi * pp[(int64_t)i * dv];   // dead (or fully underflowed) splits are not read
     }
-    float r = acc / g_sum;
     if (vB)
-      merged[idx] = r;
+      merged[idx] = acc;
     else
-      out[b * sOb + h * sOh + c] = (O)r;
+      out[b * sOb + h * sOh + c] = (O)acc;
   }
   if (!vB) return;
   __syncthreads();
@@ -240,7 +260,7 @@ template <typename O, typename TB>
 static int launch_merge(const float* partial, const float* lse, void* out, const void* vB, int64_t sVb, int64_t sVh,
                         int64_t sVr, int d_out, const int32_t* ns, const int32_t* kl, int batch, int hq, int hkv,
                         int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, hipStream_t st) {
-  size_t shm = (size_t)(hq / hkv) * dv * sizeof(float);
+  size_t shm = (size_t)(hq / hkv) * (dv + max_splits) * sizeof(float);
   merge_stage2_kernel<O, TB><<<dim3(hkv, batch), dim3(256), shm, st>>>(partial, lse, (O*)out, (const TB*)vB, sVb, sVh,
                                                                       sVr, d_out, ns, kl, hq, hkv, kv_len, max_splits,
                                                                       dv, sOb, sOh);

@@ -96,6 +96,15 @@ template <bool IS_MAX, int WIDTH> __device__ __forceinline__ float row_reduce(fl
   return x;
 }
 
+// Workgroups are dealt round-robin over the 8 XCDs (one L2 each) by linear id.  `cluster` consecutive logical ids read the
+// same token rows, so a cluster must sit on one XCD; the clusters themselves go round-robin over the XCDs, which keeps
+// ragged batches (long and short sequences, dead splits) balanced across the chip.  Grid size: xcd_grid(total, cluster).
+__device__ __forceinline__ int xcd_cluster_remap(int id, int cluster) {
+  const int xcd = id & 7, j = id >> 3;
+  return ((j / cluster) * 8 + xcd) * cluster + (j % cluster);
+}
+inline int xcd_grid(int total_wg, int cluster) { return ((total_wg / cluster + 7) & ~7) * cluster; }
+
 inline int launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? XKV_OK : (int)e;
