@@ -127,7 +127,7 @@ __global__ __launch_bounds__(256) void blockdiag_q_kernel(const T* __restrict__ 
 }
 
 // ----------------------------------------------------------------------------------------------
-// Stage 2.  One workgroup per (kv head, batch): merges the live splits of its G query heads
+// Stage 2.  One workgroup per (kv head, batch), or per (query head, batch) when there are many splits: merges the live splits of its query heads
 // (reference order: increasing split id, running max of lse), then optionally multiplies the
 // merged rank-space rows by vB[b, kh] (read once for the G heads).
 // ----------------------------------------------------------------------------------------------
@@ -136,18 +136,25 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     const float* __restrict__ partial, const float* __restrict__ lse, O* __restrict__ out,
     const TB* __restrict__ vB, int64_t sVb, int64_t sVh, int64_t sVr, int d_out,
     const int32_t* __restrict__ num_kv_splits, const int32_t* __restrict__ kv_lens,
-    int hq, int hkv, int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh) {
+    int hq, int hkv, int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, int hpw) {
   extern __shared__ float merged[];  // [G][dv], then the split weights [G][max_splits]
   __shared__ float fin[4 * 256];     // per-head-block totals of the up-projection
-  const int kh = blockIdx.x, b = blockIdx.y, G = hq / hkv;
+  // this workgroup: heads hfirst .. hfirst + G - 1 of sequence b, all of kv head kh (G = hpw divides the GQA group size)
+  const int G = hpw, hfirst = blockIdx.x * hpw, kh = hfirst / (hq / hkv), b = blockIdx.y;
   const int L = kv_lens ? kv_lens[b] : kv_len;
   const int ns = num_kv_splits[b];
   float* wts = merged + G * dv;
+  int nlive = 0;
+  {
+    const int per = ns > 0 ? cdiv(cdiv(L, ns), MIN_BLOCK_KV) * MIN_BLOCK_KV : 0;
+    nlive = per > 0 ? cdiv(L, per) : 0;
+    nlive = nlive < max_splits ? nlive : max_splits;
+  }
   // weights of the live splits, w_i = exp(lse_i - max lse) / sum: one wave per head, lanes stride over the splits
   {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int gi = wave; gi < G; gi += 4) {
-      const float* pl = lse + ((int64_t)b * hq + kh * G + gi) * max_splits;
+      const float* pl = lse + ((int64_t)b * hq + hfirst + gi) * max_splits;
       float mx = NEG_INF;
       for (int i = lane; i < max_splits; i += 64) {
         int s0, e0;
@@ -174,15 +181,13 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
   __syncthreads();
   for (int idx = threadIdx.x; idx < G * dv; idx += blockDim.x) {
     const int gi = idx / dv, c = idx - gi * dv;
-    const int h = kh * G + gi;
+    const int h = hfirst + gi;
     const float* pp = partial + ((int64_t)b * hq + h) * max_splits * (int64_t)dv + c;
     const float* w = wts + gi * max_splits;
     float acc = 0.f;
+    // live splits are a prefix (split i is live iff per * i < L): unconditional, independent loads
 #pragma unroll 8
-    for (int i = 0; i < max_splits; ++i) {
-      const float wi = w[i];
-      if (wi != 0.f) acc += wi * pp[(int64_t)i * dv];   // dead (or fully underflowed) splits are not read
-    }
+    for (int i = 0; i < nlive; ++i) acc += w[i] * pp[(int64_t)i * dv];
     if (vB)
       merged[idx] = acc;
     else
@@ -242,7 +247,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     __syncthreads();
     for (int idx = threadIdx.x; idx < 4 * d_out; idx += blockDim.x) {
       const int gi = idx / d_out, c = idx - gi * d_out;
-      if (g0 + gi < G) out[b * sOb + (kh * G + g0 + gi) * sOh + c] = (O)fin[idx];
+      if (g0 + gi < G) out[b * sOb + (hfirst + g0 + gi) * sOh + c] = (O)fin[idx];
     }
   }
 }
@@ -260,10 +265,13 @@ template <typename O, typename TB>
 static int launch_merge(const float* partial, const float* lse, void* out, const void* vB, int64_t sVb, int64_t sVh,
                         int64_t sVr, int d_out, const int32_t* ns, const int32_t* kl, int batch, int hq, int hkv,
                         int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, hipStream_t st) {
-  size_t shm = (size_t)(hq / hkv) * (dv + max_splits) * sizeof(float);
-  merge_stage2_kernel<O, TB><<<dim3(hkv, batch), dim3(256), shm, st>>>(partial, lse, (O*)out, (const TB*)vB, sVb, sVh,
-                                                                      sVr, d_out, ns, kl, hq, hkv, kv_len, max_splits,
-                                                                      dv, sOb, sOh);
+  // few splits: one workgroup per kv head (vB read once for its heads); many splits: one per query head, so that the
+  // partial rows of a long sequence are spread over more CUs
+  const int hpw = max_splits > 16 ? 1 : hq / hkv;
+  size_t shm = (size_t)hpw * (dv + max_splits) * sizeof(float);
+  merge_stage2_kernel<O, TB><<<dim3(hq / hpw, batch), dim3(256), shm, st>>>(partial, lse, (O*)out, (const TB*)vB, sVb, sVh,
+                                                                           sVr, d_out, ns, kl, hq, hkv, kv_len, max_splits,
+                                                                           dv, sOb, sOh, hpw);
   return launch_status();
 }
 
