@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define XKV_ABI_VERSION 1
+#define XKV_ABI_VERSION 2
 
 enum { XKV_F16 = 0, XKV_BF16 = 1, XKV_F32 = 2 };
 
@@ -56,7 +56,7 @@ int xkv_rope_table(void* sin_out, void* cos_out, const float* inv_freq, int64_t 
  * Replaces the host-side torch.matmul(q_nope, kv_B_nope.transpose(1, 2)) at
  * flash_decoding/mla2/mla_flash_decoding.py:81-82 and is what makes the no-PE score scan a GEMV
  * over A (the eager form attention.py:312-318) instead of the per-tile reconstruction of
- * flash_recontruction/qAB_no_pe/v1.py:53-74.   d <= 256, d % 8 == 0. */
+ * flash_recontruction/qAB_no_pe/v1.py:53-74.   d <= 512, d % 8 == 0. */
 int xkv_absorb_q(const void* q, const void* B, void* qt_hi, void* qt_lo,
                  int batch, int hq, int hkv, int d, int rank,
                  int64_t stride_B_b, int64_t stride_B_h, int64_t stride_B_r,
@@ -154,13 +154,17 @@ int64_t xkv_recon_workspace_bytes(int batch, int hkv, int rank, int64_t stride_k
  * (stride_o_b, stride_o_h), written as out_dtype.
  * Replaces _fwd_kernel_stage2[grid] at flash_decoding/gqa.py:322-337 (mla.py, mla2/stage2.py:117-135,
  * fused_attention/no_pe/v1.py:345-362 twins) and the torch.matmul with v_B_buffer at
- * fused_attention/no_pe/v2.py:468-471 / v1.py:458-460.   dv <= 512; d_out <= 256. */
+ * fused_attention/no_pe/v2.py:468-471 / v1.py:458-460.   dv <= 512; d_out <= 256.
+ * lse_out (may be NULL): the log-sum-exp of the merged range, lse_out[b * stride_lse_b + h * stride_lse_h] =
+ * log sum_i exp(lse_i), which lets the merged row take part in a further merge as one split (prefix + tail decode,
+ * flash_decoding/deepseek_mla/flash_decoding.py:137-155 concatenates the workspaces instead). */
 int xkv_merge_stage2(const float* partial, const float* lse, void* out,
                      const void* vB, int64_t stride_vB_b, int64_t stride_vB_h, int64_t stride_vB_r,
                      int d_out, int vB_dtype,
                      const int32_t* num_kv_splits, const int32_t* kv_lens,
                      int batch, int hq, int hkv, int kv_len, int max_splits, int dv,
-                     int64_t stride_o_b, int64_t stride_o_h, int out_dtype, void* stream);
+                     int64_t stride_o_b, int64_t stride_o_h, int out_dtype,
+                     float* lse_out, int64_t stride_lse_b, int64_t stride_lse_h, void* stream);
 
 #ifdef __cplusplus
 }

@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("XKV_HIP_LIB", os.path.join(_HERE, "libxkv_hip.so"))  # override: another build of the same ABI
 
 XKV_F16, XKV_BF16, XKV_F32 = 0, 1, 2
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 EXPORTS = (
     "xkv_abi_version", "xkv_error_string", "xkv_rope_table", "xkv_absorb_q",
@@ -58,7 +58,7 @@ def _declare(lib):
     lib.xkv_merge_stage2.restype = c_int
     lib.xkv_merge_stage2.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                     c_int64, c_int64, c_int, c_void_p]
+                                     c_int64, c_int64, c_int, c_void_p, c_int64, c_int64, c_void_p]
 
 
 def lib():

@@ -33,11 +33,15 @@ __global__ __launch_bounds__(256) void absorb_q_kernel(
     int hq, int hkv, int d, int rank, int64_t sBb, int64_t sBh, int64_t sBr) {
   typedef typename Elem<T>::vec8 vec8;
   __shared__ float qs[32 * 256];
-  const int kh = blockIdx.x, b = blockIdx.y, G = hq / hkv;
-  const T* qb = q + ((int64_t)b * hq + (int64_t)kh * G) * d;
+  const int kh = blockIdx.x, b = blockIdx.y, Gall = hq / hkv;
+  const int HC = 8192 / d < 32 ? 8192 / d : 32;   // heads whose query rows fit the LDS buffer at a time
+  const T* Bh = B + b * sBb + kh * sBh;
+  for (int gc = 0; gc < Gall; gc += HC) {
+  const int G = Gall - gc < HC ? Gall - gc : HC;
+  const T* qb = q + ((int64_t)b * hq + (int64_t)kh * Gall + gc) * d;
+  __syncthreads();
   for (int i = threadIdx.x; i < G * d; i += blockDim.x) qs[i] = to_f32(qb[i]);
   __syncthreads();
-  const T* Bh = B + b * sBb + kh * sBh;
   for (int rho = blockIdx.z * blockDim.x + threadIdx.x; rho < rank; rho += blockDim.x * gridDim.z) {
     const T* row = Bh + rho * sBr;
     for (int g0 = 0; g0 < G; g0 += 4) {
@@ -55,51 +59,59 @@ __global__ __launch_bounds__(256) void absorb_q_kernel(
 #pragma unroll
       for (int gi = 0; gi < 4; ++gi)
         if (g0 + gi < G) {
-          int64_t o = ((int64_t)b * hq + (int64_t)kh * G + g0 + gi) * rank + rho;
+          int64_t o = ((int64_t)b * hq + (int64_t)kh * Gall + gc + g0 + gi) * rank + rho;
           T hi = from_f32<T>(acc[gi]);
           qt_hi[o] = hi;
           if (qt_lo) qt_lo[o] = from_f32<T>(acc[gi] - to_f32(hi));
         }
     }
   }
+  }
 }
 
-// Same product for head_dim 64 / 128 with coalesced reads: TPR = d / 8 consecutive lanes cover one row of B (16 bytes
-// each), 256 / TPR rows per pass, 64 rows per workgroup; the per-row dot products are finished by a DPP reduction.
+// Same product for head_dim 64 / 128 / 256 / 512 with coalesced reads: TPR = d / 8 consecutive lanes cover one row of B
+// (16 bytes each), 256 / TPR rows per pass, 64 rows per workgroup; the per-row dot products are finished by a lane
+// reduction.  The query rows sit in LDS as fp32, 8192 values (HC = 8192 / d heads) at a time.
 template <typename T, int TPR>
 __global__ __launch_bounds__(256) void absorb_q_rows_kernel(
     const T* __restrict__ q, const T* __restrict__ B, T* __restrict__ qt_hi, T* __restrict__ qt_lo,
     int hq, int hkv, int rank, int64_t sBb, int64_t sBh, int64_t sBr) {
   typedef typename Elem<T>::vec8 vec8;
-  constexpr int D = TPR * 8, RPP = 256 / TPR;
-  __shared__ float qs[32 * D];
+  constexpr int D = TPR * 8, RPP = 256 / TPR, HC = 8192 / D < 32 ? 8192 / D : 32;
+  __shared__ float qs[HC * D];
   const int kh = blockIdx.x, b = blockIdx.y, G = hq / hkv;
-  const T* qb = q + ((int64_t)b * hq + (int64_t)kh * G) * D;
-  for (int i = threadIdx.x; i < G * D; i += 256) qs[i] = to_f32(qb[i]);
-  __syncthreads();
   const int sub = threadIdx.x % TPR, rr = threadIdx.x / TPR;
   const T* Bh = B + b * sBb + kh * sBh;
-  for (int r0 = 0; r0 < 64; r0 += RPP) {
-    const int rho = blockIdx.z * 64 + r0 + rr;
-    const bool live = rho < rank;
-    float x[8];
-    {
-      vec8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (live) v = ld16<vec8>(Bh + (int64_t)rho * sBr + sub * 8);
+  for (int g0 = 0; g0 < G; g0 += HC) {
+    const int gn = G - g0 < HC ? G - g0 : HC;
+    const T* qb = q + ((int64_t)b * hq + (int64_t)kh * G + g0) * D;
+    __syncthreads();
+    for (int i = threadIdx.x; i < gn * D; i += 256) qs[i] = to_f32(qb[i]);
+    __syncthreads();
+    for (int r0 = 0; r0 < 64; r0 += RPP) {
+      const int rho = blockIdx.z * 64 + r0 + rr;
+      const bool live = rho < rank;
+      float x[8];
+      {
+        vec8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (live) v = ld16<vec8>(Bh + (int64_t)rho * sBr + sub * 8);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) x[e] = to_f32(v[e]);
-    }
-    for (int g = 0; g < G; ++g) {
-      const f32x4 qa = *reinterpret_cast<const f32x4*>(qs + g * D + sub * 8);
-      const f32x4 qb4 = *reinterpret_cast<const f32x4*>(qs + g * D + sub * 8 + 4);
-      float a = x[0] * qa[0] + x[1] * qa[1] + x[2] * qa[2] + x[3] * qa[3] + x[4] * qb4[0] + x[5] * qb4[1] + x[6] * qb4[2] +
-                x[7] * qb4[3];
-      a = row_reduce<false, TPR>(a);
-      if (live && sub == (g % TPR)) {
-        const int64_t o = ((int64_t)b * hq + (int64_t)kh * G + g) * rank + rho;
-        const T hi = from_f32<T>(a);
-        qt_hi[o] = hi;
-        if (qt_lo) qt_lo[o] = from_f32<T>(a - to_f32(hi));
+        for (int e = 0; e < 8; ++e) x[e] = to_f32(v[e]);
+      }
+      for (int g = 0; g < gn; ++g) {
+        const f32x4 qa = *reinterpret_cast<const f32x4*>(qs + g * D + sub * 8);
+        const f32x4 qb4 = *reinterpret_cast<const f32x4*>(qs + g * D + sub * 8 + 4);
+        float a = x[0] * qa[0] + x[1] * qa[1] + x[2] * qa[2] + x[3] * qa[3] + x[4] * qb4[0] + x[5] * qb4[1] +
+                  x[6] * qb4[2] + x[7] * qb4[3];
+        a = row_reduce<false, (TPR < 16 ? TPR : 16)>(a);
+        if (TPR >= 32) a += __shfl_xor(a, 16);
+        if (TPR >= 64) a += __shfl_xor(a, 32);
+        if (live && sub == (g % TPR)) {
+          const int64_t o = ((int64_t)b * hq + (int64_t)kh * G + g0 + g) * rank + rho;
+          const T hi = from_f32<T>(a);
+          qt_hi[o] = hi;
+          if (qt_lo) qt_lo[o] = from_f32<T>(a - to_f32(hi));
+        }
       }
     }
   }
@@ -136,7 +148,8 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     const float* __restrict__ partial, const float* __restrict__ lse, O* __restrict__ out,
     const TB* __restrict__ vB, int64_t sVb, int64_t sVh, int64_t sVr, int d_out,
     const int32_t* __restrict__ num_kv_splits, const int32_t* __restrict__ kv_lens,
-    int hq, int hkv, int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, int hpw) {
+    int hq, int hkv, int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, int hpw,
+    float* __restrict__ lse_out, int64_t sLb, int64_t sLh) {
   extern __shared__ float merged[];  // [G][dv], then the split weights [G][max_splits]
   __shared__ float fin[4 * 256];     // per-head-block totals of the up-projection
   // this workgroup: heads hfirst .. hfirst + G - 1 of sequence b, all of kv head kh (G = hpw divides the GQA group size)
@@ -176,6 +189,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
       for (int o = 1; o < 64; o <<= 1) sum += __shfl_xor(sum, o);
       const float inv = 1.f / sum;
       for (int i = lane; i < max_splits; i += 64) wts[gi * max_splits + i] *= inv;
+      if (lse_out && lane == 0) lse_out[b * sLb + (hfirst + gi) * sLh] = mx + __logf(sum);   // log-sum-exp of the merged range
     }
   }
   __syncthreads();
@@ -264,14 +278,15 @@ static int launch_rope(void* s, void* c, const float* inv, int64_t seqlen, int64
 template <typename O, typename TB>
 static int launch_merge(const float* partial, const float* lse, void* out, const void* vB, int64_t sVb, int64_t sVh,
                         int64_t sVr, int d_out, const int32_t* ns, const int32_t* kl, int batch, int hq, int hkv,
-                        int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, hipStream_t st) {
+                        int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, float* lse_out, int64_t sLb, int64_t sLh,
+                        hipStream_t st) {
   // few splits: one workgroup per kv head (vB read once for its heads); many splits: one per query head, so that the
   // partial rows of a long sequence are spread over more CUs
-  const int hpw = max_splits > 16 ? 1 : hq / hkv;
+  const int hpw = (max_splits > 16 || hq / hkv > 16) ? 1 : hq / hkv;
   size_t shm = (size_t)hpw * (dv + max_splits) * sizeof(float);
   merge_stage2_kernel<O, TB><<<dim3(hq / hpw, batch), dim3(256), shm, st>>>(partial, lse, (O*)out, (const TB*)vB, sVb, sVh,
                                                                            sVr, d_out, ns, kl, hq, hkv, kv_len, max_splits,
-                                                                           dv, sOb, sOh, hpw);
+                                                                           dv, sOb, sOh, hpw, lse_out, sLb, sLh);
   return launch_status();
 }
 
@@ -308,7 +323,7 @@ extern "C" int xkv_rope_table(void* sin_out, void* cos_out, const float* inv_fre
 extern "C" int xkv_absorb_q(const void* q, const void* B, void* qt_hi, void* qt_lo, int batch, int hq, int hkv, int d,
                             int rank, int64_t sBb, int64_t sBh, int64_t sBr, int dtype, void* stream) {
   if (!q || !B || !qt_hi || batch <= 0 || hq <= 0 || hkv <= 0 || d <= 0 || rank <= 0) return XKV_EINVAL;
-  if (hq % hkv || hq / hkv > 32 || d > 256 || d % 8) return XKV_EUNSUPPORTED;
+  if (hq % hkv || hq / hkv > 32 || d > 512 || d % 8) return XKV_EUNSUPPORTED;
   if (sBr % 8 || sBh % 8 || sBb % 8 || ((uintptr_t)B & 15)) return XKV_EALIGN;
   hipStream_t st = (hipStream_t)stream;
   if (dtype != XKV_BF16 && dtype != XKV_F16) return XKV_EDTYPE;
@@ -316,6 +331,12 @@ extern "C" int xkv_absorb_q(const void* q, const void* B, void* qt_hi, void* qt_
 #define XKV_ABSORB(T)                                                                                                         \
   if (d == 128)                                                                                                               \
     absorb_q_rows_kernel<T, 16><<<dim3(hkv, batch, (rank + 63) / 64), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,    \
+                                                                                        (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr); \
+  else if (d == 512)                                                                                                          \
+    absorb_q_rows_kernel<T, 64><<<dim3(hkv, batch, (rank + 63) / 64), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,    \
+                                                                                        (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr); \
+  else if (d == 256)                                                                                                          \
+    absorb_q_rows_kernel<T, 32><<<dim3(hkv, batch, (rank + 63) / 64), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,    \
                                                                                         (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr); \
   else if (d == 64)                                                                                                           \
     absorb_q_rows_kernel<T, 8><<<dim3(hkv, batch, (rank + 63) / 64), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,     \
@@ -344,14 +365,15 @@ extern "C" int xkv_blockdiag_q(const void* q, void* out, int batch, int hq, int 
 extern "C" int xkv_merge_stage2(const float* partial, const float* lse, void* out, const void* vB, int64_t sVb,
                                 int64_t sVh, int64_t sVr, int d_out, int vB_dtype, const int32_t* ns,
                                 const int32_t* kl, int batch, int hq, int hkv, int kv_len, int max_splits, int dv,
-                                int64_t sOb, int64_t sOh, int out_dtype, void* stream) {
+                                int64_t sOb, int64_t sOh, int out_dtype, float* lse_out, int64_t sLb, int64_t sLh,
+                                void* stream) {
   if (!partial || !lse || !out || !ns || batch <= 0 || hq <= 0 || hkv <= 0 || max_splits <= 0 || dv <= 0)
     return XKV_EINVAL;
-  if (hq % hkv || hq / hkv > 16 || dv > 512) return XKV_EUNSUPPORTED;
+  if (hq % hkv || hq / hkv > 32 || dv > 512) return XKV_EUNSUPPORTED;
   if (vB && (d_out <= 0 || d_out > 256 || d_out % 8)) return XKV_EUNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
 #define XKV_MERGE(O, TB) \
-  return launch_merge<O, TB>(partial, lse, out, vB, sVb, sVh, sVr, d_out, ns, kl, batch, hq, hkv, kv_len, max_splits, dv, sOb, sOh, st)
+  return launch_merge<O, TB>(partial, lse, out, vB, sVb, sVh, sVr, d_out, ns, kl, batch, hq, hkv, kv_len, max_splits, dv, sOb, sOh, lse_out, sLb, sLh, st)
   const int bt = vB ? vB_dtype : XKV_BF16;
   if (bt != XKV_BF16 && bt != XKV_F16) return XKV_EDTYPE;
   switch (out_dtype) {

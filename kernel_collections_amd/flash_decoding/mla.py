@@ -23,7 +23,9 @@ def _split_dims(dk: int):
     return dk, 0
 
 
-def decode_attention_fwd(q, k_buffer, v_buffer, o, sm_scale=1.0, logit_cap=0.0):
+def stage1_operands(q, k_buffer, v_buffer):
+    """Shape checks and operand descriptors shared by every entry built on this kernel:
+    returns ``(qn, qr, C, R, V, groups, dn, dv)``."""
     batch, num_q_heads, head_dim = q.shape
     _, kv_len, num_kv_heads, dk = k_buffer.shape
     assert dk == head_dim
@@ -42,12 +44,19 @@ def decode_attention_fwd(q, k_buffer, v_buffer, o, sm_scale=1.0, logit_cap=0.0):
     groups = num_kv_heads * per_kv_groups
     sh = k_buffer.stride(2) if per_kv_groups == 1 else 0
     svh = v_buffer.stride(2) if per_kv_groups == 1 else 0
-    S = ops.latent_splits(batch, groups, kv_len, dn)
-    splits = ops.uniform_splits(batch, S, q.device)
-    partial, lse = ops.workspaces(batch, num_q_heads, S, dv, q.device)
     C = (k_buffer, k_buffer.stride(0), k_buffer.stride(1), sh, dn)
     R = (k_buffer[..., dn:], k_buffer.stride(0), k_buffer.stride(1), sh, dr) if dr else None
     V = (v_buffer, v_buffer.stride(0), v_buffer.stride(1), svh, dv)
+    return qn, qr, C, R, V, groups, dn, dv
+
+
+def decode_attention_fwd(q, k_buffer, v_buffer, o, sm_scale=1.0, logit_cap=0.0):
+    batch, num_q_heads, _ = q.shape
+    kv_len = k_buffer.shape[1]
+    qn, qr, C, R, V, groups, dn, dv = stage1_operands(q, k_buffer, v_buffer)
+    S = ops.latent_splits(batch, groups, kv_len, dn)
+    splits = ops.uniform_splits(batch, S, q.device)
+    partial, lse = ops.workspaces(batch, num_q_heads, S, dv, q.device)
     ops.latent_stage1(qn, None, qr, C, R, V, partial, lse, None, splits, None, batch, num_q_heads, groups,
                       kv_len, S, float(sm_scale), float(logit_cap))
     ops.merge_stage2(partial, lse, o, None, splits, None, batch, num_q_heads, num_q_heads, kv_len, S)

@@ -60,6 +60,18 @@ def occupancy_splits(batch: int, groups: int, kv_len: int, tile: int = 64, waves
     return max(1, min(want, cap))
 
 
+def settled_splits(kv_len: int, n: int) -> int:
+    """Largest split count <= n under which EVERY split is live: with `per = cdiv(cdiv(kv_len, n), 32) * 32` tokens per
+    split only the first cdiv(kv_len, per) splits hold tokens (flash_decoding/gqa.py:95-99 of the reference)."""
+    n = max(1, int(n))
+    while True:
+        per = _cdiv(_cdiv(kv_len, n), 32) * 32
+        live = max(1, _cdiv(kv_len, per))
+        if live == n:
+            return n
+        n = live
+
+
 def latent_splits(batch: int, groups: int, kv_len: int, width: int) -> int:
     """Split count for the dot-product stage 1: 512-wide rows run the LDS-ring kernel (one workgroup per CU,
     32-token tiles), everything else the register-staged one (two workgroups per CU, 64-token tiles)."""
@@ -150,21 +162,28 @@ def recon_stage1(q3, kA, kB, vA, partial, lse, scores, num_kv_splits, kv_lens, b
         "xkv_recon_stage1")
 
 
-def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, kv_len, max_splits):
-    """out `[b,Hq,*]` (strides honoured on the first two axes)."""
+def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, kv_len, max_splits, lse_out=None):
+    """out `[b,Hq,*]` (strides honoured on the first two axes).  `lse_out` `[b,Hq]` (any strides, fp32): log-sum-exp
+    of the merged range.  Up-projections wider than 256 columns run as column blocks of 256."""
     dv = partial.shape[-1]
     assert out.stride(-1) == 1
-    if vB is not None:
-        vB = as_rows(vB)
-        sv = (vB.stride(0), vB.stride(1), vB.stride(2))
-        d_out, vdt = vB.shape[-1], dtype_code(vB.dtype)
-    else:
-        sv, d_out, vdt = (0, 0, 0), dv, _lib.XKV_BF16
-    check(_lib.lib().xkv_merge_stage2(
-        ptr(partial), ptr(lse), ptr(out), ptr(vB), c_int64(sv[0]), c_int64(sv[1]), c_int64(sv[2]), d_out, vdt,
-        ptr(num_kv_splits), ptr(kv_lens), batch, hq, hkv, kv_len, max_splits, dv,
-        c_int64(out.stride(0)), c_int64(out.stride(1)), dtype_code(out.dtype), stream_ptr(partial)),
-        "xkv_merge_stage2")
+    sl = (0, 0) if lse_out is None else (lse_out.stride(0), lse_out.stride(1))
+
+    def call(o, w, d_out, sv, vdt, lo):
+        check(_lib.lib().xkv_merge_stage2(
+            ptr(partial), ptr(lse), ptr(o), ptr(w), c_int64(sv[0]), c_int64(sv[1]), c_int64(sv[2]), d_out, vdt,
+            ptr(num_kv_splits), ptr(kv_lens), batch, hq, hkv, kv_len, max_splits, dv,
+            c_int64(o.stride(0)), c_int64(o.stride(1)), dtype_code(o.dtype), ptr(lo), c_int64(sl[0]), c_int64(sl[1]),
+            stream_ptr(partial)), "xkv_merge_stage2")
+
+    if vB is None:
+        call(out, None, dv, (0, 0, 0), _lib.XKV_BF16, lse_out)
+        return out
+    vB = as_rows(vB)
+    sv, vdt = (vB.stride(0), vB.stride(1), vB.stride(2)), dtype_code(vB.dtype)
+    for c0 in range(0, vB.shape[-1], 256):
+        c1 = min(c0 + 256, vB.shape[-1])
+        call(out[..., c0:c1], vB[..., c0:c1], c1 - c0, sv, vdt, lse_out if c0 == 0 else None)
     return out
 
 

@@ -117,3 +117,16 @@ def test_eager_surface_functions_agree_with_the_oracle():
     assert torch.equal(cos, ocos) and torch.equal(sin, osin)
     x = r(50, 128).float()
     assert torch.equal(rope_ref.apply_rotary_pos_emb_pytorch(x, cos, sin)[0], oracle.apply_rope(x, ocos, osin))
+
+
+def test_settled_splits_leaves_no_dead_split():
+    """A workspace shared by two stage-1 passes is merged as 'all rows live': the host must never ask for more splits
+    than the split arithmetic fills."""
+    import oracle
+    from kernel_collections_amd import ops
+    for L in list(range(1, 400)) + [1500, 4096, 4097, 131072]:
+        for n in (1, 2, 3, 4, 7, 11, 16, 64, 128):
+            s = ops.settled_splits(L, n)
+            assert 1 <= s <= n
+            live = oracle.live_splits(L, s, s)
+            assert len(live) == s and live[0][1] == 0 and live[-1][2] == L, (L, n, s)

@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 
 import kernel_collections_amd.flash_recontruction as fr  # noqa: E402
 from kernel_collections_amd import ops  # noqa: E402
-from kernel_collections_amd.flash_decoding import gqa, mla, mla2  # noqa: E402
+from kernel_collections_amd.flash_decoding import deepseek_mla, gqa, mla, mla2  # noqa: E402
 from kernel_collections_amd.flash_recontruction.rope.sin_cos import rotary_sin_cos  # noqa: E402
 
 BF, FP = torch.bfloat16, torch.float16
@@ -311,6 +311,43 @@ def test_mla_py_concat_layout(dev, dk, dv, hkv):
     o2 = torch.zeros_like(o)
     mla.decode_attention_fwd(q.to(dev), Kd, Vd, o2, 0.2, 30.0)
     check_out(o2, ref_c, "mla.py logit cap")
+
+
+# ------------------------------------------------------------------------------------ prefix + tail decode
+@pytest.mark.parametrize("dtype", [BF, FP])
+@pytest.mark.parametrize("b,H,hd,Lp,Ld,r", [(2, 32, 512, 1500, 100, 512),   # the reference test's shape, shortened
+                                            (1, 16, 576, 700, 33, 512),     # 512 + 64 RoPE features, tail shorter than 2 blocks
+                                            (3, 8, 128, 300, 1, 256)])      # one decoded token
+def test_prefix_tail_decode(dev, dtype, b, H, hd, Lp, Ld, r):
+    """flash_decoding/deepseek_mla: attention over [prefix | tail] computed as two stage-1 passes and one merge equals
+    plain attention over the concatenation; in the factorised form the prefix is K = k_A k_B, V = v_A v_B."""
+    scale = hd ** -0.5
+    q = gen((b, H, hd), dtype=dtype, seed=1)
+    kA, vA = gen((b, Lp, r), dtype=dtype, seed=2), gen((b, Lp, r), dtype=dtype, seed=3)
+    kB, vB = gen((b, 1, r, hd), std=r ** -0.5, dtype=dtype, seed=4), gen((b, 1, r, hd), std=r ** -0.5, dtype=dtype, seed=5)
+    Kd, Vd = gen((b, Ld, 1, hd), dtype=dtype, seed=6), gen((b, Ld, 1, hd), dtype=dtype, seed=7)
+    # the plain-buffer entry points see the prefix rounded to the operand type; the factorised one reconstructs it in fp32
+    Kp32 = oracle.reconstruct(*f32(kA, kB)).transpose(1, 2)
+    Vp32 = oracle.reconstruct(*f32(vA, vB)).transpose(1, 2)
+    Kp, Vp = Kp32.to(dtype), Vp32.to(dtype)
+    qd, kAd, vAd, kBd, vBd, Kdd, Vdd, Kpd, Vpd = dev_(dev, q, kA, vA, kB, vB, Kd, Vd, Kp, Vp)
+    if hd != 576:
+        ref_plain = oracle.gqa_plain(q.float(), torch.cat([Kp.float(), Kd.float()], 1),
+                                     torch.cat([Vp.float(), Vd.float()], 1), scale)
+        ref_xkv = oracle.gqa_plain(q.float(), torch.cat([Kp32, Kd.float()], 1), torch.cat([Vp32, Vd.float()], 1), scale)
+        o_one = deepseek_mla.mla_decode_attention_fwd(qd, torch.cat([Kpd, Kdd], 1), torch.cat([Vpd, Vdd], 1), scale)
+        check_out(o_one, ref_plain, "one buffer")
+        o_sep = deepseek_mla.mla_decode_attention_fwd_pd_sep(qd, Kpd, Vpd, Kdd, Vdd, scale)
+        check_out(o_sep, ref_plain, "prefix + tail, plain")
+        assert max_abs(o_sep, o_one) < 4e-3, "splitting the buffer in two must not change the result beyond rounding"
+        if hd <= 256 or hd == 512:
+            o_x = deepseek_mla.mla_decode_attention_fwd_pd_sep_xKV(qd, kAd, kBd, vAd, vBd, Kdd, Vdd, scale)
+            check_out(o_x, ref_xkv, "prefix factorised + tail plain")
+    else:
+        # MLA layout: a 576-wide key buffer whose first 512 features are also the values
+        o_sep = deepseek_mla.mla_decode_attention_fwd_pd_sep(qd, Kpd, Kpd[..., :512], Kdd, Kdd[..., :512], scale)
+        Kall = torch.cat([Kp.float(), Kd.float()], 1)
+        check_out(o_sep, oracle.gqa_plain(q.float(), Kall, Kall[..., :512], scale), "prefix + tail, MLA layout")
 
 
 # ------------------------------------------------------------------------------------ split handling, bit-exact
