@@ -279,12 +279,41 @@ def bench_c4(args, dev, vfact):
     }
 
 
+def bench_pdsep(args, dev):
+    """Prefix + tail decode at the shape of the reference's own script (test_mla_decoding_new.py:66-73): batch 1,
+    32 heads on one kv head, head_dim 512, prefix 262144 tokens factorised at rank 512, 128 decoded tokens, fp16."""
+    from kernel_collections_amd.flash_decoding import deepseek_mla
+    B, H, hd, Lp, Ld, r = 1, 32, 512, 262144, 128, 512
+    dt = torch.float16
+    gen = torch.Generator(device=dev).manual_seed(0)
+    q = randn_dev((B, H, hd), 1.0, dev, dt, gen)
+    kA, vA = randn_dev((B, Lp, r), 1.0, dev, dt, gen), randn_dev((B, Lp, r), 1.0, dev, dt, gen)
+    kB, vB = randn_dev((B, 1, r, hd), r ** -0.5, dev, dt, gen), randn_dev((B, 1, r, hd), r ** -0.5, dev, dt, gen)
+    Kd, Vd = randn_dev((B, Ld, 1, hd), 1.0, dev, dt, gen), randn_dev((B, Ld, 1, hd), 1.0, dev, dt, gen)
+    scale = hd ** -0.5
+    fn = lambda i: deepseek_mla.mla_decode_attention_fwd_pd_sep_xKV(q, kA, kB, vA, vB, Kd, Vd, scale)
+    total_ms = time_loop(fn, args.steps, args.warmup)
+    us = total_ms * 1e3 / args.steps
+    algo_bytes = B * Lp * 2 * r * 2 + B * Ld * 2 * hd * 2 + 2 * r * hd * 2
+    gbs = algo_bytes / (us * 1e-6) / 1e9
+    return {
+        "metric": "us_per_prefix_tail_decode_step", "value": round(us, 2), "unit": "us", "higher_is_better": False,
+        "ms_per_step": total_ms / args.steps,
+        "config": {"workload": "prefix + tail decode: batch 1, 32 heads / 1 kv head, head_dim 512, prefix 262144 at rank 512 "
+                               "(k_A, v_A), tail 128 plain, fp16"},
+        "roofline": {"bound": "hbm", "kernel": "latent_ring_kernel", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None,
+                     "note": "whole call (absorb, 2 x stage 1, 2 x merge) over algorithmic bytes", "algorithmic_bytes": algo_bytes},
+        "cpu_baseline": None,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=25)
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c4v", "c5"])
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c4v", "c5", "pdsep"])
     ap.add_argument("--ctx", type=int, default=32768)
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
@@ -312,12 +341,14 @@ def main():
         res = bench_c2(args, dev)
     elif args.config == "c5":
         res = bench_c5(args, dev)
+    elif args.config == "pdsep":
+        res = bench_pdsep(args, dev)
     else:
         res = bench_c4(args, dev, args.config == "c4v")
     line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"), "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": res.pop("ms_per_step"),
             "higher_is_better": res.pop("higher_is_better"), "scaling": "weak", "vs_baseline": None,
-            "dtype": "bf16", "data": "synthetic"}
+            "dtype": "fp16" if args.config == "pdsep" else "bf16", "data": "synthetic"}
     line.update(res)
     print(json.dumps(line))
 

@@ -154,7 +154,7 @@ int64_t xkv_recon_workspace_bytes(int batch, int hkv, int rank, int64_t stride_k
  * (stride_o_b, stride_o_h), written as out_dtype.
  * Replaces _fwd_kernel_stage2[grid] at flash_decoding/gqa.py:322-337 (mla.py, mla2/stage2.py:117-135,
  * fused_attention/no_pe/v1.py:345-362 twins) and the torch.matmul with v_B_buffer at
- * fused_attention/no_pe/v2.py:468-471 / v1.py:458-460.   dv <= 512; d_out <= 256.
+ * fused_attention/no_pe/v2.py:468-471 / v1.py:458-460.   dv <= 512; d_out <= 512.
  * lse_out (may be NULL): the log-sum-exp of the merged range, lse_out[b * stride_lse_b + h * stride_lse_h] =
  * log sum_i exp(lse_i), which lets the merged row take part in a further merge as one split (prefix + tail decode,
  * flash_decoding/deepseek_mla/flash_decoding.py:137-155 concatenates the workspaces instead). */

@@ -70,48 +70,47 @@ __global__ __launch_bounds__(256) void absorb_q_kernel(
 }
 
 // Same product for head_dim 64 / 128 / 256 / 512 with coalesced reads: TPR = d / 8 consecutive lanes cover one row of B
-// (16 bytes each), 256 / TPR rows per pass, 64 rows per workgroup; the per-row dot products are finished by a lane
-// reduction.  The query rows sit in LDS as fp32, 8192 values (HC = 8192 / d heads) at a time.
+// (16 bytes each), 256 / TPR rows per pass; the per-row dot products are finished by a lane reduction.  A workgroup
+// takes ABS_ROWS rows of B and up to ABS_HEADS query heads of one kv head (their rows sit in LDS as fp32), so that
+// even a single sequence with one kv head spreads over tens of CUs.
+constexpr int ABS_ROWS = 16, ABS_HEADS = 8;
 template <typename T, int TPR>
 __global__ __launch_bounds__(256) void absorb_q_rows_kernel(
     const T* __restrict__ q, const T* __restrict__ B, T* __restrict__ qt_hi, T* __restrict__ qt_lo,
-    int hq, int hkv, int rank, int64_t sBb, int64_t sBh, int64_t sBr) {
+    int hq, int hkv, int rank, int64_t sBb, int64_t sBh, int64_t sBr, int nhc) {
   typedef typename Elem<T>::vec8 vec8;
-  constexpr int D = TPR * 8, RPP = 256 / TPR, HC = 8192 / D < 32 ? 8192 / D : 32;
-  __shared__ float qs[HC * D];
-  const int kh = blockIdx.x, b = blockIdx.y, G = hq / hkv;
+  constexpr int D = TPR * 8, RPP = 256 / TPR;
+  __shared__ float qs[ABS_HEADS * D];
+  const int kh = blockIdx.x / nhc, g0 = (blockIdx.x % nhc) * ABS_HEADS, b = blockIdx.y, G = hq / hkv;
+  const int gn = G - g0 < ABS_HEADS ? G - g0 : ABS_HEADS;
   const int sub = threadIdx.x % TPR, rr = threadIdx.x / TPR;
   const T* Bh = B + b * sBb + kh * sBh;
-  for (int g0 = 0; g0 < G; g0 += HC) {
-    const int gn = G - g0 < HC ? G - g0 : HC;
-    const T* qb = q + ((int64_t)b * hq + (int64_t)kh * G + g0) * D;
-    __syncthreads();
-    for (int i = threadIdx.x; i < gn * D; i += 256) qs[i] = to_f32(qb[i]);
-    __syncthreads();
-    for (int r0 = 0; r0 < 64; r0 += RPP) {
-      const int rho = blockIdx.z * 64 + r0 + rr;
-      const bool live = rho < rank;
-      float x[8];
-      {
-        vec8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (live) v = ld16<vec8>(Bh + (int64_t)rho * sBr + sub * 8);
+  const T* qb = q + ((int64_t)b * hq + (int64_t)kh * G + g0) * D;
+  for (int i = threadIdx.x; i < gn * D; i += 256) qs[i] = to_f32(qb[i]);
+  __syncthreads();
+  for (int r0 = 0; r0 < ABS_ROWS; r0 += RPP) {
+    const int rho = blockIdx.z * ABS_ROWS + r0 + rr;
+    const bool live = rho < rank && rr < ABS_ROWS;
+    float x[8];
+    {
+      vec8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (live) v = ld16<vec8>(Bh + (int64_t)rho * sBr + sub * 8);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = to_f32(v[e]);
-      }
-      for (int g = 0; g < gn; ++g) {
-        const f32x4 qa = *reinterpret_cast<const f32x4*>(qs + g * D + sub * 8);
-        const f32x4 qb4 = *reinterpret_cast<const f32x4*>(qs + g * D + sub * 8 + 4);
-        float a = x[0] * qa[0] + x[1] * qa[1] + x[2] * qa[2] + x[3] * qa[3] + x[4] * qb4[0] + x[5] * qb4[1] +
-                  x[6] * qb4[2] + x[7] * qb4[3];
-        a = row_reduce<false, (TPR < 16 ? TPR : 16)>(a);
-        if (TPR >= 32) a += __shfl_xor(a, 16);
-        if (TPR >= 64) a += __shfl_xor(a, 32);
-        if (live && sub == (g % TPR)) {
-          const int64_t o = ((int64_t)b * hq + (int64_t)kh * G + g0 + g) * rank + rho;
-          const T hi = from_f32<T>(a);
-          qt_hi[o] = hi;
-          if (qt_lo) qt_lo[o] = from_f32<T>(a - to_f32(hi));
-        }
+      for (int e = 0; e < 8; ++e) x[e] = to_f32(v[e]);
+    }
+    for (int g = 0; g < gn; ++g) {
+      const f32x4 qa = *reinterpret_cast<const f32x4*>(qs + g * D + sub * 8);
+      const f32x4 qb4 = *reinterpret_cast<const f32x4*>(qs + g * D + sub * 8 + 4);
+      float a = x[0] * qa[0] + x[1] * qa[1] + x[2] * qa[2] + x[3] * qa[3] + x[4] * qb4[0] + x[5] * qb4[1] +
+                x[6] * qb4[2] + x[7] * qb4[3];
+      a = row_reduce<false, (TPR < 16 ? TPR : 16)>(a);
+      if (TPR >= 32) a += __shfl_xor(a, 16);
+      if (TPR >= 64) a += __shfl_xor(a, 32);
+      if (live && sub == (g % TPR)) {
+        const int64_t o = ((int64_t)b * hq + (int64_t)kh * G + g0 + g) * rank + rho;
+        const T hi = from_f32<T>(a);
+        qt_hi[o] = hi;
+        if (qt_lo) qt_lo[o] = from_f32<T>(a - to_f32(hi));
       }
     }
   }
@@ -151,7 +150,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     int hq, int hkv, int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, int hpw,
     float* __restrict__ lse_out, int64_t sLb, int64_t sLh) {
   extern __shared__ float merged[];  // [G][dv], then the split weights [G][max_splits]
-  __shared__ float fin[4 * 256];     // per-head-block totals of the up-projection
+  __shared__ float fin[4 * 512];     // per-head-block totals of the up-projection
   // this workgroup: heads hfirst .. hfirst + G - 1 of sequence b, all of kv head kh (G = hpw divides the GQA group size)
   const int G = hpw, hfirst = blockIdx.x * hpw, kh = hfirst / (hq / hkv), b = blockIdx.y;
   const int L = kv_lens ? kv_lens[b] : kv_len;
@@ -214,7 +213,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
   typedef typename Elem<TB>::vec8 vec8;
   const TB* Bh = vB + b * sVb + kh * sVh;
   __shared__ float red[32 * 4 * 64];                 // [rank group][4 heads][columns of the block]  (<= 32 KiB)
-  const int ncb = (d_out + 7) >> 3;                  // 8-column blocks (d_out <= 256 -> <= 32)
+  const int ncb = (d_out + 7) >> 3;                  // 8-column blocks (d_out <= 512 -> <= 64)
   const int ngrp = 256 / ncb;                        // rank groups
   const int cb = threadIdx.x % ncb, grp = threadIdx.x / ncb;
   const bool active = grp < ngrp && cb * 8 + 8 <= d_out;
@@ -237,8 +236,8 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
       }
     }
     // reduce over the rank groups through LDS, `chunk` groups per pass (as many as fit `red`)
-    const int cols = ncb * 8;                        // <= 256
-    const int chunk = 32 * 64 / cols;                // >= 8
+    const int cols = ncb * 8;                        // <= 512
+    const int chunk = 32 * 64 / cols;                // >= 4
     for (int base = 0; base < ngrp; base += chunk) {
       __syncthreads();
       if (active && grp >= base && grp < base + chunk) {
@@ -328,19 +327,20 @@ extern "C" int xkv_absorb_q(const void* q, const void* B, void* qt_hi, void* qt_
   hipStream_t st = (hipStream_t)stream;
   if (dtype != XKV_BF16 && dtype != XKV_F16) return XKV_EDTYPE;
   const dim3 block(256);
+  const int nhc = (hq / hkv + ABS_HEADS - 1) / ABS_HEADS;   // head chunks per kv head
 #define XKV_ABSORB(T)                                                                                                         \
   if (d == 128)                                                                                                               \
-    absorb_q_rows_kernel<T, 16><<<dim3(hkv, batch, (rank + 63) / 64), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,    \
-                                                                                        (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr); \
+    absorb_q_rows_kernel<T, 16><<<dim3(hkv * nhc, batch, (rank + ABS_ROWS - 1) / ABS_ROWS), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,    \
+                                                                                        (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr, nhc); \
   else if (d == 512)                                                                                                          \
-    absorb_q_rows_kernel<T, 64><<<dim3(hkv, batch, (rank + 63) / 64), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,    \
-                                                                                        (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr); \
+    absorb_q_rows_kernel<T, 64><<<dim3(hkv * nhc, batch, (rank + ABS_ROWS - 1) / ABS_ROWS), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,    \
+                                                                                        (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr, nhc); \
   else if (d == 256)                                                                                                          \
-    absorb_q_rows_kernel<T, 32><<<dim3(hkv, batch, (rank + 63) / 64), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,    \
-                                                                                        (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr); \
+    absorb_q_rows_kernel<T, 32><<<dim3(hkv * nhc, batch, (rank + ABS_ROWS - 1) / ABS_ROWS), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,    \
+                                                                                        (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr, nhc); \
   else if (d == 64)                                                                                                           \
-    absorb_q_rows_kernel<T, 8><<<dim3(hkv, batch, (rank + 63) / 64), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,     \
-                                                                                       (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr); \
+    absorb_q_rows_kernel<T, 8><<<dim3(hkv * nhc, batch, (rank + ABS_ROWS - 1) / ABS_ROWS), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi,     \
+                                                                                       (T*)qt_lo, hq, hkv, rank, sBb, sBh, sBr, nhc); \
   else                                                                                                                        \
     absorb_q_kernel<T><<<dim3(hkv, batch, (rank + 255) / 256), block, 0, st>>>((const T*)q, (const T*)B, (T*)qt_hi, (T*)qt_lo, \
                                                                                  hq, hkv, d, rank, sBb, sBh, sBr);
@@ -370,7 +370,7 @@ extern "C" int xkv_merge_stage2(const float* partial, const float* lse, void* ou
   if (!partial || !lse || !out || !ns || batch <= 0 || hq <= 0 || hkv <= 0 || max_splits <= 0 || dv <= 0)
     return XKV_EINVAL;
   if (hq % hkv || hq / hkv > 32 || dv > 512) return XKV_EUNSUPPORTED;
-  if (vB && (d_out <= 0 || d_out > 256 || d_out % 8)) return XKV_EUNSUPPORTED;
+  if (vB && (d_out <= 0 || d_out > 512 || d_out % 8)) return XKV_EUNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
 #define XKV_MERGE(O, TB) \
   return launch_merge<O, TB>(partial, lse, out, vB, sVb, sVh, sVr, d_out, ns, kl, batch, hq, hkv, kv_len, max_splits, dv, sOb, sOh, lse_out, sLb, sLh, st)

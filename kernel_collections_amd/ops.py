@@ -164,7 +164,7 @@ def recon_stage1(q3, kA, kB, vA, partial, lse, scores, num_kv_splits, kv_lens, b
 
 def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, kv_len, max_splits, lse_out=None):
     """out `[b,Hq,*]` (strides honoured on the first two axes).  `lse_out` `[b,Hq]` (any strides, fp32): log-sum-exp
-    of the merged range.  Up-projections wider than 256 columns run as column blocks of 256."""
+    of the merged range.  Up-projections wider than 512 columns run as column blocks of 512."""
     dv = partial.shape[-1]
     assert out.stride(-1) == 1
     sl = (0, 0) if lse_out is None else (lse_out.stride(0), lse_out.stride(1))
@@ -181,8 +181,8 @@ def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, 
         return out
     vB = as_rows(vB)
     sv, vdt = (vB.stride(0), vB.stride(1), vB.stride(2)), dtype_code(vB.dtype)
-    for c0 in range(0, vB.shape[-1], 256):
-        c1 = min(c0 + 256, vB.shape[-1])
+    for c0 in range(0, vB.shape[-1], 512):
+        c1 = min(c0 + 512, vB.shape[-1])
         call(out[..., c0:c1], vB[..., c0:c1], c1 - c0, sv, vdt, lse_out if c0 == 0 else None)
     return out
 
