@@ -6,8 +6,10 @@
 // (HBM latency x its share of the HBM rate) = 60-100 KB of loads in flight to stream at full rate, which a
 // register-staged double buffer cannot hold.  Here the token rows go HBM -> LDS directly
 // (global_load_lds_dwordx4, no VGPRs involved) into a ring of RSLOT tiles of TN tokens, RSLOT-1 tiles always in
-// flight, one workgroup per CU, and the query operands live in registers for the whole kernel, so the per-tile work is
-//   A:  wait for tile t, barrier, issue tile t+RSLOT-1 into the slot PV(t-1) just released
+// flight, one workgroup per CU, and the query operands live in registers for the whole kernel.  The loads are issued by
+// two extra wavefronts that do nothing else (a load instruction that stalls on a full memory queue then never holds up
+// the arithmetic); they take part in the same barriers.  Per tile:
+//   A:  loaders wait for tile t; barrier; loaders issue tile t+RSLOT-1 into the slot PV(t-1) just released
 //   QK: wave (tb, kh) multiplies token block tb by its k-range kh of q on v_mfma_f32_16x16x32 -> partial scores in LDS
 //   B:  barrier; softmax threads add the k-range partials, update the running max / sum, publish P and alpha
 //   C:  barrier; PV: each wave owns a quarter of the value features, token-major operand via ds_read_b64_tr_b16.
@@ -67,8 +69,8 @@ struct RingShape {
 // T: operand type; TN: tokens per tile (32, or 16 when two row streams share the LDS); NHB: 16-row head blocks; LO: q has
 // a low-order part; DN: latent width; HAS_R: 64 RoPE features follow (TN 32 only); VMODE: scores only / V is the first
 // 512 features of the C row / V is a second 512-wide row stream.
-template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE>
-__global__ __launch_bounds__(256) void latent_ring_kernel(const RingParams p) {
+template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE, int NLOAD>
+__global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const RingParams p) {
   typedef typename Elem<T>::vec8 vec8;
   typedef RingShape<TN, DN, HAS_R, VMODE, NHB> S;
   constexpr bool SCORES = VMODE == RING_SCORES;
@@ -79,8 +81,13 @@ __global__ __launch_bounds__(256) void latent_ring_kernel(const RingParams p) {
   static_assert(NKS % KSPLIT == 0, "the k-ranges are equal");
   static_assert(!HAS_R || TN == 32, "RoPE-key rows need 32-token tiles");
   constexpr int IPR = DN / 512;                   // 1 KiB load instructions per C row
-  constexpr int RPW = TN / 4;                     // rows per wave per tile
-  constexpr int LPT = RPW * IPR + (HAS_R ? 1 : 0) + (VMODE == RING_VDISTINCT ? RPW : 0);   // loads per wave per tile
+  // who issues the tile loads: the four compute waves (NLOAD == 0) or NLOAD extra waves that do nothing else, so that a
+  // load instruction stalled on a full memory queue never holds up the MFMA / softmax work
+  constexpr int NISS = NLOAD ? NLOAD : 4;
+  constexpr int RPW = TN / NISS;                  // rows per issuing wave per tile
+  constexpr int RIW = 4 / NISS;                   // RoPE-key load instructions per issuing wave (4 per tile)
+  constexpr int LPT = RPW * IPR + (HAS_R ? RIW : 0) + (VMODE == RING_VDISTINCT ? RPW : 0);   // loads per issuing wave per tile
+  constexpr int WAITN = (RSLOT - 2) * LPT < 63 ? (RSLOT - 2) * LPT : 63;   // vmcnt holds 6 bits
   constexpr int DV = 512, NVB = DV / 64;          // value features, 16-feature blocks per wave
   constexpr int TPH = 256 / HB, TPT = TN / TPH;   // softmax threads per head row, tokens per thread
   static_assert(TPT >= 1, "tile too short for the softmax thread map");
@@ -90,6 +97,7 @@ __global__ __launch_bounds__(256) void latent_ring_kernel(const RingParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n16 = lane & 15, g4 = lane >> 4;
   const int tb = wave % NTB, kh = wave / NTB;
+  const int iw = NLOAD ? wave - 4 : wave;         // index among the issuing waves (negative: not an issuer)
 
   const int wg = xcd_cluster_remap(blockIdx.x, p.groups);   // the kv groups of one (sequence, split) share an L2
   if (wg >= p.total_wg) return;
@@ -119,24 +127,24 @@ __global__ __launch_bounds__(256) void latent_ring_kernel(const RingParams p) {
       VMODE == RING_VDISTINCT ? reinterpret_cast<const unsigned char*>(p.V) + (b * p.sVb + group * p.sVh) * 2 : nullptr;
   const int64_t crow_bytes = p.sCl * 2, rrow_bytes = p.sRl * 2, vrow_bytes = p.sVl * 2;
   const unsigned lane_off = lane * 16;
-  const int r_row = lane & 31, r_chunk = 2 * wave + (lane >> 5);
+  const int r_row = lane & 31;
   auto issue_tile = [&](int t) {
     const unsigned slot = ring_lds + (unsigned)(t % RSLOT) * SLOT;
     const int base = start + t * TN;
-    const int tok0 = base + wave * RPW;
+    const int tok0 = base + iw * RPW;
     if (base + TN <= end) {            // whole tile inside the split: row pointers advance by adds
       const unsigned char* row = Cb + (int64_t)tok0 * crow_bytes;
 #pragma unroll
       for (int r = 0; r < RPW; ++r) {
 #pragma unroll
-        for (int c = 0; c < IPR; ++c) ring_load16(row + c * 1024, lane_off, slot + (wave * RPW + r) * CROW + c * 1024);
+        for (int c = 0; c < IPR; ++c) ring_load16(row + c * 1024, lane_off, slot + (iw * RPW + r) * CROW + c * 1024);
         row += crow_bytes;
       }
       if (VMODE == RING_VDISTINCT) {
         const unsigned char* vrow = Vb + (int64_t)tok0 * vrow_bytes;
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
-          ring_load16(vrow, lane_off, slot + CBYTES + S::RBYTES + (wave * RPW + r) * VROW);
+          ring_load16(vrow, lane_off, slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW);
           vrow += vrow_bytes;
         }
       }
@@ -147,19 +155,36 @@ __global__ __launch_bounds__(256) void latent_ring_kernel(const RingParams p) {
         tok = tok < last ? tok : last;   // rows past the split end are masked in the softmax; keep the read in bounds
         const unsigned char* row = Cb + (int64_t)tok * crow_bytes;
 #pragma unroll
-        for (int c = 0; c < IPR; ++c) ring_load16(row + c * 1024, lane_off, slot + (wave * RPW + r) * CROW + c * 1024);
+        for (int c = 0; c < IPR; ++c) ring_load16(row + c * 1024, lane_off, slot + (iw * RPW + r) * CROW + c * 1024);
         if (VMODE == RING_VDISTINCT)
-          ring_load16(Vb + (int64_t)tok * vrow_bytes, lane_off, slot + CBYTES + S::RBYTES + (wave * RPW + r) * VROW);
+          ring_load16(Vb + (int64_t)tok * vrow_bytes, lane_off, slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW);
       }
     }
     if (HAS_R) {
       int tok = base + r_row;
       tok = tok < last ? tok : last;
-      ring_load16(Rb, (unsigned)tok * (unsigned)rrow_bytes + r_chunk * 16, slot + CBYTES + wave * 1024);
+#pragma unroll
+      for (int j = 0; j < RIW; ++j) {   // instruction w of 4 brings chunks 2w, 2w+1 of every row
+        const int w = iw * RIW + j;
+        ring_load16(Rb, (unsigned)tok * (unsigned)rrow_bytes + (2 * w + (lane >> 5)) * 16, slot + CBYTES + w * 1024);
+      }
     }
   };
+  if (iw >= 0) {
 #pragma unroll
-  for (int t = 0; t < RSLOT - 1; ++t) issue_tile(t);
+    for (int t = 0; t < RSLOT - 1; ++t) issue_tile(t);
+  }
+  if (NLOAD && wave >= 4) {            // loader wave: keep RSLOT-1 tiles in flight, take part in every barrier of the loop
+    for (int t = 0; t < ntiles; ++t) {
+      ring_wait<WAITN>();              // tile t has landed
+      __syncthreads();                 // A
+      issue_tile(t + RSLOT - 1);
+      __syncthreads();                 // B
+      if (!SCORES) __syncthreads();    // C
+    }
+    ring_wait<0>();
+    return;
+  }
 
   // ---- query operands in registers: lane (n16 = head row, g4) holds q[head][32 ks + 8 g4 .. +8] for its k-range ----
   vec8 qreg[KS_W][NHB], qlo[LO ? KS_W : 1][NHB];
@@ -206,9 +231,9 @@ __global__ __launch_bounds__(256) void latent_ring_kernel(const RingParams p) {
   const int vcol0 = wave * (DV / 4);
 
   for (int t = 0; t < ntiles; ++t) {
-    ring_wait<(RSLOT - 2) * LPT>();   // this wave's rows of tile t have landed (RSLOT-2 younger tiles may be in flight)
+    if (!NLOAD) ring_wait<WAITN>();   // this wave's rows of tile t have landed (RSLOT-2 younger tiles may be in flight)
     __syncthreads();                  // A: tile t complete for every wave; every wave is past PV / score write of tile t-1
-    issue_tile(t + RSLOT - 1);        // into the slot of tile t-1 (past the end: clamped rows, never used)
+    if (!NLOAD) issue_tile(t + RSLOT - 1);   // into the slot of tile t-1 (past the end: clamped rows, never used)
     const unsigned char* slot = ring + (t % RSLOT) * SLOT;
     const int base = start + t * TN;
 
@@ -333,7 +358,7 @@ __global__ __launch_bounds__(256) void latent_ring_kernel(const RingParams p) {
       }
     }
   }
-  ring_wait<0>();                     // drain the clamped look-ahead loads before the workgroup's LDS is released
+  if (!NLOAD) ring_wait<0>();         // drain the clamped look-ahead loads before the workgroup's LDS is released
   if (SCORES) return;
 
   // ---- epilogue: normalise, write partial + lse --------------------------------------------------------------------
@@ -354,14 +379,18 @@ __global__ __launch_bounds__(256) void latent_ring_kernel(const RingParams p) {
   }
 }
 
+#ifndef XKV_RING_NLOAD
+#define XKV_RING_NLOAD 2
+#endif
 template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE>
 static int launch_ring_t(const RingParams& p, int batch, hipStream_t st) {
   constexpr int SHM = RingShape<TN, DN, HAS_R, VMODE, NHB>::SHM;
-  auto kern = latent_ring_kernel<T, TN, NHB, LO, DN, HAS_R, VMODE>;
+  constexpr int NLOAD = XKV_RING_NLOAD;
+  auto kern = latent_ring_kernel<T, TN, NHB, LO, DN, HAS_R, VMODE, NLOAD>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SHM);
   if (e != hipSuccess) return (int)e;
   const int total = batch * p.groups * p.max_splits;
-  kern<<<dim3(xcd_grid(total, p.groups)), dim3(256), SHM, st>>>(p);
+  kern<<<dim3(xcd_grid(total, p.groups)), dim3(256 + 64 * NLOAD), SHM, st>>>(p);
   return launch_status();
 }
 
