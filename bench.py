@@ -28,7 +28,7 @@ PEAK_BF16_TFLOPS = 2500.0
 # HBM bytes of one stage-1 launch at the default c3 shape, from two rocprofv3 --pmc runs of this file
 # (FETCH_SIZE, WRITE_SIZE; each scaled by what the counter reads for --calib-copy's 512 MiB copies).
 # A counter cannot be read from inside the timed process, so the figure is recorded here.
-C3_STAGE1_HBM_BYTES = 535259 * 1024
+C3_STAGE1_HBM_BYTES = 535406 * 1024
 
 
 def _events(n):
