@@ -350,6 +350,39 @@ def test_prefix_tail_decode(dev, dtype, b, H, hd, Lp, Ld, r):
         check_out(o_sep, oracle.gqa_plain(q.float(), Kall, Kall[..., :512], scale), "prefix + tail, MLA layout")
 
 
+# ------------------------------------------------------------------------------------ committed vectors
+def test_committed_golden_vectors(dev):
+    """The HIP path on the committed inputs (tests/golden/xkv_vectors.npz; all values exactly representable in bf16)
+    against the committed oracle outputs."""
+    import os
+    import numpy as np
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "xkv_vectors.npz"), allow_pickle=False)
+    g = {k: torch.from_numpy(z[k]) for k in z.files}
+    h = lambda k: g[k].to(BF).to(dev)
+    q, A, Av, kB, vB, K, V = (h(k) for k in ("q", "A", "Av", "kB", "vB", "K", "V"))
+    theta, scale = float(g["theta"]), float(g["scale"])
+    b, hq = q.shape[0], q.shape[1]
+    S = 2
+    ns = splits_t([S] * b, dev)
+    check_scores(fr.qAB_no_pe_v1(q, A, kB, out_dtype=torch.float32), g["qab_nope"], "qab_nope")
+    check_scores(fr.qAB_rope_v1(q, A, kB, theta, out_dtype=torch.float32), g["qab_rope"], "qab_rope")
+    q3 = q[:, :, 0].contiguous()
+    check_out(fr.gqa_xKV_no_pe_v2(q3, A, kB, Av, vB, ns, S, scale), g["gqa_xkv"], "gqa_xkv")
+    o = torch.empty_like(q3)
+    fr.gqa_xKV_rope(q3, A, kB, Av, vB, o, ns, S, scale, theta)
+    check_out(o, g["gqa_factorized_rope"], "gqa_factorized_rope")
+    o = torch.empty_like(q3)
+    gqa.decode_attention_fwd(q3, K, V, o, ns, S, scale)
+    check_out(o, g["gqa_plain"], "gqa_plain")
+    o = torch.empty_like(q3)
+    gqa.decode_attention_fwd_v_factorized(q3, K, Av, vB, o, ns, S, scale)
+    check_out(o, g["gqa_v_only"], "gqa_v_only")
+    sin, cos = rotary_sin_cos(A.shape[1], theta, 0, device=dev)
+    assert max_abs(torch.cat((sin, cos), -1), g["sin_cos_table"]) < 2e-6
+    out = mla2.mla_decode_attention_fwd(h("mla_qn"), h("mla_qr"), h("mla_ckv"), h("mla_kpe"), float(g["mla_scale"]))
+    check_out(out, g["mla_ref"], "mla_ref")
+
+
 # ------------------------------------------------------------------------------------ split handling, bit-exact
 @pytest.mark.parametrize("L,ns,S", [(1000, 4, 4), (100, 8, 8), (4096, 3, 5), (33, 2, 2), (64, 1, 3)])
 def test_split_index_handling_is_exact(dev, L, ns, S):
