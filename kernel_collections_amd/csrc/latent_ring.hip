@@ -263,31 +263,32 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
     __syncthreads();                  // B: the k-range partials of every head row are visible
 
     if (SCORES) {
-      // thread -> head row tid / (TN/8), tokens 8 (tid % (TN/8)) .. +8: a 32-byte piece of a score row
-      constexpr int PPR = TN / 8;
-      const int row = tid / PPR, c0 = (tid % PPR) * 8;
-      if (row < hg) {
-        const int64_t o = ((int64_t)b * p.hq + h0 + row) * p.kv_len + base + c0;
-        float s[8];
+      // thread -> 4 tokens (16 bytes) of a head row, TN/4 consecutive lanes per row: every store instruction writes whole
+      // 128-byte (TN 32) pieces of score rows; rows beyond the first 256 / (TN/4) come in a second pass
+      constexpr int LPR = TN / 4, RPP = 256 / LPR;
+      const int c0 = (tid % LPR) * 4;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          float a = 0.f;
+      for (int row = tid / LPR; row < HB; row += RPP) {
+        if (row < hg) {
+          const int64_t o = ((int64_t)b * p.hq + h0 + row) * p.kv_len + base + c0;
+          f32x4 a = *reinterpret_cast<const f32x4*>(s_part + row * SP + c0);
 #pragma unroll
-          for (int kr = 0; kr < KSPLIT; ++kr) a += s_part[(kr * HB + row) * SP + c0 + j];
-          s[j] = a * p.sm_scale;
-          if (p.logit_cap > 0.f) s[j] = p.logit_cap * tanhf(s[j] / p.logit_cap);
-        }
-        if (p.scores_dtype == XKV_F32 && (p.kv_len & 3) == 0 && base + c0 + 8 <= end) {
-          float* dst = reinterpret_cast<float*>(p.scores) + o;
-          *reinterpret_cast<f32x4*>(dst) = f32x4{s[0], s[1], s[2], s[3]};
-          *reinterpret_cast<f32x4*>(dst + 4) = f32x4{s[4], s[5], s[6], s[7]};
-        } else {
+          for (int kr = 1; kr < KSPLIT; ++kr) a += *reinterpret_cast<const f32x4*>(s_part + (kr * HB + row) * SP + c0);
+          a *= p.sm_scale;
+          if (p.logit_cap > 0.f) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j)
-            if (base + c0 + j < end) {
-              if (p.scores_dtype == XKV_F32) reinterpret_cast<float*>(p.scores)[o + j] = s[j];
-              else reinterpret_cast<T*>(p.scores)[o + j] = from_f32<T>(s[j]);
-            }
+            for (int j = 0; j < 4; ++j) a[j] = p.logit_cap * tanhf(a[j] / p.logit_cap);
+          }
+          if (p.scores_dtype == XKV_F32 && (p.kv_len & 3) == 0 && base + c0 + 4 <= end) {
+            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.scores) + o) = a;
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (base + c0 + j < end) {
+                if (p.scores_dtype == XKV_F32) reinterpret_cast<float*>(p.scores)[o + j] = a[j];
+                else reinterpret_cast<T*>(p.scores)[o + j] = from_f32<T>(a[j]);
+              }
+          }
         }
       }
       continue;

@@ -44,7 +44,8 @@ def test_rope_table(dev, theta, start):
 # ------------------------------------------------------------------------------------ qAB, no PE
 @pytest.mark.parametrize("dtype", [BF, FP])
 @pytest.mark.parametrize("b,hq,hkv,L,r", [(2, 32, 8, 1000, 512), (1, 8, 8, 77, 192), (3, 16, 2, 4133, 256),
-                                          (1, 64, 8, 300, 384), (2, 4, 1, 64, 64)])
+                                          (1, 64, 8, 300, 384), (2, 4, 1, 64, 64),
+                                          (1, 32, 8, 5, 512), (2, 16, 2, 33, 512)])   # shorter than one tile / one token over
 def test_qab_nope(dev, dtype, b, hq, hkv, L, r):
     d = 128
     q, A, B = gen((b, hq, 1, d), dtype=dtype, seed=1), gen((b, L, r), dtype=dtype, seed=2), \
@@ -108,7 +109,8 @@ def test_qab_rope_long_positions(dev):
 # ------------------------------------------------------------------------------------ fused xKV decode, no PE
 @pytest.mark.parametrize("dtype", [BF, FP])
 @pytest.mark.parametrize("b,hq,hkv,L,rk,rv,S", [(2, 32, 8, 3000, 256, 384, 8), (1, 32, 8, 700, 512, 512, 3),
-                                                (3, 8, 8, 129, 192, 64, 2), (1, 16, 4, 4096, 384, 256, 16)])
+                                                (3, 8, 8, 129, 192, 64, 2), (1, 16, 4, 4096, 384, 256, 16),
+                                                (2, 32, 8, 40, 512, 512, 2), (1, 8, 2, 3, 512, 512, 4)])   # fewer live splits than asked
 def test_fused_nope(dev, dtype, b, hq, hkv, L, rk, rv, S):
     d = 128
     q = gen((b, hq, d), std=1 / 3, dtype=dtype, seed=1)
@@ -265,8 +267,9 @@ def test_blockdiag_q_is_exact(dev):
 
 # ------------------------------------------------------------------------------------ MLA
 @pytest.mark.parametrize("dtype", [BF, FP])
-def test_mla2(dev, dtype):
-    b, H, L, c, e = 3, 16, 2100, 512, 64
+@pytest.mark.parametrize("L", [2100, 17])
+def test_mla2(dev, dtype, L):
+    b, H, c, e = 3, 16, 512, 64
     qn, qr = gen((b, H, c), std=1 / 3, dtype=dtype, seed=1), gen((b, H, e), std=1 / 3, dtype=dtype, seed=2)
     ckv, kpe = gen((b, L, 1, c), std=1 / 3, dtype=dtype, seed=3), gen((b, L, 1, e), std=1 / 3, dtype=dtype, seed=4)
     scale = 1 / math.sqrt(192)
