@@ -56,6 +56,19 @@ __device__ __forceinline__ void async_row16(const void* row_base, unsigned lane_
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_off), "s"(row_base)
                : "memory", "m0");
 }
+// Four rows with one M0 / base pair: the instruction offset r * FROW moves the LDS address AND the global address, so the
+// per-row lane offsets voff[r] = lane * 16 + 128 + r * (row_bytes - FROW) (base = first row - 128 bytes) put row r of the
+// tile at global row r.  (FROW must stay below 4096 / 3 for the 13-bit offset field.)
+__device__ __forceinline__ void async_rows4(const void* base_m128, unsigned v0, unsigned v1, unsigned v2, unsigned v3,
+                                            unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+               "global_load_lds_dwordx4 %1, %5\n\t"
+               "global_load_lds_dwordx4 %2, %5 offset:1040\n\t"
+               "global_load_lds_dwordx4 %3, %5 offset:2080\n\t"
+               "global_load_lds_dwordx4 %4, %5 offset:3120"
+               ::"s"(lds_addr), "v"(v0), "v"(v1), "v"(v2), "v"(v3), "s"(base_m128)
+               : "memory", "m0");
+}
 template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -123,17 +136,18 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   const unsigned char* Ab = reinterpret_cast<const unsigned char*>(p.kA) + b * p.sAb * 2;
   const int64_t row_bytes = p.sAl * 2;
   const unsigned lane_off = lane * 16;
+  unsigned voff4[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) voff4[r] = lane_off + 128u + (unsigned)(r * ((int)row_bytes - FROW));
   auto issue_rows = [&](int t, auto r0_c, auto r1_c, auto full_c) {   // rows r0 .. r1-1 of this wave's 8 rows of tile t
     constexpr int R0 = decltype(r0_c)::value, R1 = decltype(r1_c)::value;
     const unsigned dst = ring_lds + (unsigned)(t & (FRING - 1)) * FTILE + (unsigned)(wave * 8) * FROW;
     const int tok0 = start + t * FT + wave * 8;
     if (decltype(full_c)::value) {   // the caller knows the whole tile lies inside the split
-      const unsigned char* row = Ab + (int64_t)(tok0 + R0) * row_bytes;
+      static_assert(!decltype(full_c)::value || ((R1 - R0) % 4 == 0 && R0 % 4 == 0), "full tiles are issued four rows at a time");
 #pragma unroll
-      for (int r = R0; r < R1; ++r) {
-        async_row16(row, lane_off, dst + r * FROW);
-        row += row_bytes;
-      }
+      for (int r = R0; r < R1; r += 4)
+        async_rows4(Ab + (int64_t)(tok0 + r) * row_bytes - 128, voff4[0], voff4[1], voff4[2], voff4[3], dst + r * FROW);
     } else {
 #pragma unroll
       for (int r = R0; r < R1; ++r) {
@@ -400,9 +414,8 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
         if (u == 4) at_next[5] = tile_frag(i + 1, 5);
         qop_next[u - 1] = ld16<vec8>(qrow + (u - 1) * 32);
         recon_step(11 + u);
-        if (u == 1) issue_rows(i + 3, IC<0>(), IC<3>(), full_c);   // into the ring slot of tile i-1, whose readers are done
-        if (u == 2) issue_rows(i + 3, IC<3>(), IC<6>(), full_c);
-        if (u == 3) issue_rows(i + 3, IC<6>(), IC<8>(), full_c);
+        if (u == 1) issue_rows(i + 3, IC<0>(), IC<4>(), full_c);   // into the ring slot of tile i-1, whose readers are done
+        if (u == 3) issue_rows(i + 3, IC<4>(), IC<8>(), full_c);
         if (u == 4) write_qhat(i + 1);                             // buffer (i+1)&1 was last read in part 3 of iteration i-1
       }
       XKV_FENCE();
