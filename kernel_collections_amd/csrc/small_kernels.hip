@@ -192,19 +192,60 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     }
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < G * dv; idx += blockDim.x) {
-    const int gi = idx / dv, c = idx - gi * dv;
-    const int h = hfirst + gi;
-    const float* pp = partial + ((int64_t)b * hq + h) * max_splits * (int64_t)dv + c;
-    const float* w = wts + gi * max_splits;
-    float acc = 0.f;
-    // live splits are a prefix (split i is live iff per * i < L): unconditional, independent loads
+  // weighted sum of the live splits (a prefix of the split range: split i is live iff per * i < L), 16 bytes per load.
+  // Work item = 4 consecutive features of one head; when there are fewer items than threads the threads form split
+  // groups (split i goes to group i % nsg) whose sums meet in LDS, so that a single long sequence still has 256 loads
+  // in flight per workgroup.
+  if ((dv & 3) == 0 && (reinterpret_cast<uintptr_t>(partial) & 15) == 0) {
+    const int items = G * dv / 4;
+    const int lanes_per = items < 256 ? items : 256;
+    const int nsg = 256 / lanes_per, sg = threadIdx.x / lanes_per;
+    for (int item = threadIdx.x % lanes_per; item < items && sg < nsg; item += lanes_per) {
+      const int gi = (item * 4) / dv, c = item * 4 - gi * dv;
+      const int h = hfirst + gi;
+      const float* pp = partial + ((int64_t)b * hq + h) * max_splits * (int64_t)dv + c;
+      const float* w = wts + gi * max_splits;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll 8
-    for (int i = 0; i < nlive; ++i) acc += w[i] * pp[(int64_t)i * dv];
-    if (vB)
-      merged[idx] = acc;
-    else
-      out[b * sOb + h * sOh + c] = (O)acc;
+      for (int i = sg; i < nlive; i += nsg) acc += w[i] * *reinterpret_cast<const f32x4*>(pp + (int64_t)i * dv);
+      if (nsg == 1) {
+        if (vB) {
+          *reinterpret_cast<f32x4*>(merged + item * 4) = acc;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out[b * sOb + h * sOh + c + e] = (O)acc[e];
+        }
+      } else {
+        *reinterpret_cast<f32x4*>(fin + (sg * items + item) * 4) = acc;   // nsg * items * 4 <= 1024 floats
+      }
+    }
+    if (nsg > 1) {
+      __syncthreads();
+      for (int idx = threadIdx.x; idx < G * dv; idx += blockDim.x) {
+        const int gi = idx / dv, c = idx - gi * dv;
+        float acc = 0.f;
+        for (int k = 0; k < nsg; ++k) acc += fin[k * items * 4 + idx];
+        if (vB)
+          merged[idx] = acc;
+        else
+          out[b * sOb + (hfirst + gi) * sOh + c] = (O)acc;
+      }
+      __syncthreads();   // fin is reused by the up-projection
+    }
+  } else {
+    for (int idx = threadIdx.x; idx < G * dv; idx += blockDim.x) {
+      const int gi = idx / dv, c = idx - gi * dv;
+      const int h = hfirst + gi;
+      const float* pp = partial + ((int64_t)b * hq + h) * max_splits * (int64_t)dv + c;
+      const float* w = wts + gi * max_splits;
+      float acc = 0.f;
+#pragma unroll 8
+      for (int i = 0; i < nlive; ++i) acc += w[i] * pp[(int64_t)i * dv];
+      if (vB)
+        merged[idx] = acc;
+      else
+        out[b * sOb + h * sOh + c] = (O)acc;
+    }
   }
   if (!vB) return;
   __syncthreads();
