@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the xKV compressed-KV decode path on one MI355X.
 
-Default workload (BASELINE config 3): fused RoPE-aware xKV decode, Llama-3.1-8B attention shape,
+Default workload (configuration 3 of the five target shapes): fused RoPE-aware xKV decode, Llama-3.1-8B attention shape,
 batch 16, 32 q / 8 kv heads, head_dim 128, context 32768, rank 512, bf16; one token basis A shared by
 K and V and by the 4 layers of a group, per-layer B_l / B_v,l.  A "step" is ONE layer's decode step
 (stage 1 + merge) cycling through the 4 layers of the group.

@@ -175,7 +175,7 @@ def test_fused_rope(dev, dtype, b, hq, hkv, L, rk, rv, S, shared):
 
 
 def test_config1_shape_factorized_rope(dev):
-    """BASELINE config 1 (batch 1, 32/8 heads, d 128, L 4096, rank 256, theta 5e5, query at 4096)."""
+    """Target configuration 1 (batch 1, 32/8 heads, d 128, L 4096, rank 256, theta 5e5, query at 4096)."""
     torch.manual_seed(0)
     b, hq, hkv, d, L, r, theta = 1, 32, 8, 128, 4096, 256, 5e5
     q = torch.randn(b, hq, 1, d)
@@ -430,7 +430,7 @@ def test_split_count_invariance_and_v1_v2_order(dev):
 
 # ------------------------------------------------------------------------------------ full-size properties
 def test_full_size_config3_properties(dev):
-    """BASELINE config 3 shape (batch 16, L 32768, rank 512) is too big for the CPU oracle as a whole:
+    """Target configuration 3 shape (batch 16, L 32768, rank 512) is too big for the CPU oracle as a whole:
     check one sequence against the oracle, and the rest through size-independent properties -
     batch permutation equivariance and linearity in v_B."""
     b, hq, hkv, d, L, r, theta = 16, 32, 8, 128, 32768, 512, 5e5
