@@ -309,14 +309,41 @@ def bench_pdsep(args, dev):
     }
 
 
+def bench_qabrope(args, dev):
+    """RoPE-aware key reconstruction scores at the shape of the reference's own sweep (test_qAB_rope.py:85-125):
+    batch 1, 32 q / 8 kv heads, head_dim 128, rank 192, fp16, kv_len = --ctx (the sweep runs 16K .. 128K)."""
+    import kernel_collections_amd.flash_recontruction as fr
+    B, Hq, Hkv, d, r, L, theta = 1, 32, 8, 128, args.rank, args.ctx, 1e7
+    dt = torch.float16
+    gen = torch.Generator(device=dev).manual_seed(0)
+    q = randn_dev((B, Hq, 1, d), 0.2, dev, dt, gen)
+    A = randn_dev((B, L, r), 0.2, dev, dt, gen)
+    Bk = randn_dev((B, Hkv, r, d), 0.2, dev, dt, gen)
+    total_ms = time_loop(lambda i: fr.qAB_rope_v1(q, A, Bk, theta), args.steps, args.warmup)
+    us = total_ms * 1e3 / args.steps
+    flops = B * L * (2 * r * Hkv * d + 2 * Hq * d)
+    tf = flops / (us * 1e-6) / 1e12
+    return {
+        "metric": "us_per_qAB_rope_call", "value": round(us, 2), "unit": "us", "higher_is_better": False,
+        "ms_per_step": total_ms / args.steps,
+        "config": {"workload": "qAB with RoPE, scores only: batch 1, 32q/8kv, d128, rank %d, kv_len %d, fp16" % (r, L)},
+        "roofline": {"bound": "mfma", "kernel": "recon_stage1_kernel(scores)", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "note": "whole call over algorithmic FLOP", "algorithmic_flop": flops,
+                     "hbm_side_GBps": round((B * L * r * 2 + B * Hq * L * 2) / (us * 1e-6) / 1e9, 1)},
+        "cpu_baseline": None,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=25)
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c4v", "c5", "pdsep"])
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c4v", "c5", "pdsep", "qabrope"])
     ap.add_argument("--ctx", type=int, default=32768)
     ap.add_argument("--splits", type=int, default=0)
+    ap.add_argument("--rank", type=int, default=192, help="rank of the qabrope workload")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-comparator", action="store_true")
     ap.add_argument("--calib-copy", action="store_true",
@@ -344,12 +371,14 @@ def main():
         res = bench_c5(args, dev)
     elif args.config == "pdsep":
         res = bench_pdsep(args, dev)
+    elif args.config == "qabrope":
+        res = bench_qabrope(args, dev)
     else:
         res = bench_c4(args, dev, args.config == "c4v")
     line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"), "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": res.pop("ms_per_step"),
             "higher_is_better": res.pop("higher_is_better"), "scaling": "weak", "vs_baseline": None,
-            "dtype": "fp16" if args.config == "pdsep" else "bf16", "data": "synthetic"}
+            "dtype": "fp16" if args.config in ("pdsep", "qabrope") else "bf16", "data": "synthetic"}
     line.update(res)
     print(json.dumps(line))
 

@@ -344,11 +344,15 @@ static int dispatch_recon(const ReconParams& p, int batch, bool vshared, hipStre
     return vshared ? launch_recon<T, 16, true, 8, true, false>(p, batch, st)
                    : launch_recon<T, 16, true, 8, false, false>(p, batch, st);
   }
-  if (p.rank == 256) {
-    if (so) return launch_recon<T, 8, true, 8, true, true>(p, batch, st);
-    return vshared ? launch_recon<T, 8, true, 8, true, false>(p, batch, st)
-                   : launch_recon<T, 8, true, 8, false, false>(p, batch, st);
+#define XKV_RECON_RANK(R)                                                                      \
+  if (p.rank == R) {                                                                           \
+    if (so) return launch_recon<T, R / 32, true, 8, true, true>(p, batch, st);                 \
+    return vshared ? launch_recon<T, R / 32, true, 8, true, false>(p, batch, st)               \
+                   : launch_recon<T, R / 32, true, 8, false, false>(p, batch, st);             \
   }
+  // exact instantiations (no per-k-step bound checks, registers sized to the rank) for the common ranks
+  XKV_RECON_RANK(384) XKV_RECON_RANK(256) XKV_RECON_RANK(192) XKV_RECON_RANK(128)
+#undef XKV_RECON_RANK
   if (so) return launch_recon<T, 16, false, 8, true, true>(p, batch, st);
   return vshared ? launch_recon<T, 16, false, 8, true, false>(p, batch, st)
                  : launch_recon<T, 16, false, 8, false, false>(p, batch, st);
