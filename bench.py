@@ -314,7 +314,7 @@ def bench_qabrope(args, dev):
     batch 1, 32 q / 8 kv heads, head_dim 128, rank 192, fp16, kv_len = --ctx (the sweep runs 16K .. 128K)."""
     import kernel_collections_amd.flash_recontruction as fr
     B, Hq, Hkv, d, r, L, theta = 1, 32, 8, 128, args.rank, args.ctx, 1e7
-    dt = torch.float16
+    dt = torch.float16 if args.dtype == "fp16" else torch.bfloat16
     gen = torch.Generator(device=dev).manual_seed(0)
     q = randn_dev((B, Hq, 1, d), 0.2, dev, dt, gen)
     A = randn_dev((B, L, r), 0.2, dev, dt, gen)
@@ -326,7 +326,7 @@ def bench_qabrope(args, dev):
     return {
         "metric": "us_per_qAB_rope_call", "value": round(us, 2), "unit": "us", "higher_is_better": False,
         "ms_per_step": total_ms / args.steps,
-        "config": {"workload": "qAB with RoPE, scores only: batch 1, 32q/8kv, d128, rank %d, kv_len %d, fp16" % (r, L)},
+        "config": {"workload": "qAB with RoPE, scores only: batch 1, 32q/8kv, d128, rank %d, kv_len %d, %s" % (r, L, args.dtype)},
         "roofline": {"bound": "mfma", "kernel": "recon_stage1_kernel(scores)", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
                      "note": "whole call over algorithmic FLOP", "algorithmic_flop": flops,
@@ -344,6 +344,7 @@ def main():
     ap.add_argument("--ctx", type=int, default=32768)
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--rank", type=int, default=192, help="rank of the qabrope workload")
+    ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16"], help="operand type of the qabrope workload")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-comparator", action="store_true")
     ap.add_argument("--calib-copy", action="store_true",
@@ -378,7 +379,7 @@ def main():
     line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"), "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": res.pop("ms_per_step"),
             "higher_is_better": res.pop("higher_is_better"), "scaling": "weak", "vs_baseline": None,
-            "dtype": "fp16" if args.config in ("pdsep", "qabrope") else "bf16", "data": "synthetic"}
+            "dtype": "fp16" if (args.config == "pdsep" or (args.config == "qabrope" and args.dtype == "fp16")) else "bf16", "data": "synthetic"}
     line.update(res)
     print(json.dumps(line))
 

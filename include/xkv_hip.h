@@ -123,7 +123,7 @@ int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_operand qr,
  * then either scores_out (as above) or the split softmax with V = vA (rank-space partials
  * [batch, hq, max_splits, vA.dim]).  rope == 0 skips the rotation (pure reconstruction).
  * Envelope: head_dim == 128, G = hq/hkv <= 16, rank % 32 == 0, rank <= 512, vA.dim % 64 == 0 <= 512.
- * With rank == 512, vA the same tensor as kA, computed angles (sin_cos == NULL), G <= 8 and a workspace of
+ * With rank == 512, scores_out or vA the same tensor as kA, computed angles (sin_cos == NULL), G <= 8 and a workspace of
  * xkv_recon_workspace_bytes() the call runs the specialised kernel (kB packed once into the workspace, 2 x 2
  * rank/feature wave split on v_mfma_f32_32x32x16, async direct-to-LDS tile ring); otherwise the generic one.
  * Replaces _qAB_fwd[grid] at flash_recontruction/qAB/v1.py:135-145 (v3.py / v4.py / ref.py twins) and

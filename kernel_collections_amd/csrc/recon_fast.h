@@ -9,6 +9,7 @@ struct FastParams {
   const void* q; const void* kA; const void* Bp;   // Bp: kB re-packed into MFMA operand order (caller workspace)
   int64_t sAb, sAl, sBpb;
   float* partial; float* lse;
+  void* scores; int scores_dtype;               // scores != NULL: write [batch, hq, kv_len] scaled scores, no softmax / P.A
   const int32_t* num_splits; const int32_t* kv_lens;
   int hq, hkv, kv_len, max_splits, total_wg;
   float sm_scale;

@@ -97,7 +97,8 @@ template <int V> using IC = std::integral_constant<int, V>;
 #define XKV_FENCE() __builtin_amdgcn_sched_barrier(0)
 #define XKV_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)   // 0x8 MFMA, 0x2 VALU, 0x100 LDS read, 0x200 LDS write
 
-template <typename T>
+// SCORES: write the scaled scores (the qAB-with-RoPE form) instead of running softmax and P.A
+template <typename T, bool SCORES>
 __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   typedef typename Elem<T>::vec8 vec8;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -238,6 +239,23 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     float s0 = (sp_v[0][0] + sp_v[1][0]) + (sp_v[2][0] + sp_v[3][0]);
     float s1 = (sp_v[0][1] + sp_v[1][1]) + (sp_v[2][1] + sp_v[3][1]);
     const int tok = start + t * FT + 2 * n16;
+    if (SCORES) {   // lanes 0..31 of wave w hold heads w and w + 4, two tokens each
+      if (sm_valid && lane < 32) {
+        const int64_t o = ((int64_t)b * p.hq + h0 + sm_head) * p.kv_len + tok;
+        s0 *= p.sm_scale;
+        s1 *= p.sm_scale;
+        if (p.scores_dtype == XKV_F32) {
+          float* dst = reinterpret_cast<float*>(p.scores) + o;
+          if (tok < end) dst[0] = s0;
+          if (tok + 1 < end) dst[1] = s1;
+        } else {
+          T* dst = reinterpret_cast<T*>(p.scores) + o;
+          if (tok < end) dst[0] = from_f32<T>(s0);
+          if (tok + 1 < end) dst[1] = from_f32<T>(s1);
+        }
+      }
+      return;
+    }
     s0 = tok < end ? s0 * p.sm_scale : NEG_INF;
     s1 = tok + 1 < end ? s1 * p.sm_scale : NEG_INF;
     // the reference maximum only moves when the tile maximum exceeds it by LAZY_RESCALE (branch-free: alpha = 1 otherwise)
@@ -344,6 +362,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     const unsigned char* vt =
         ring + ((i - 1) & (FRING - 1)) * FTILE + (8 * g4 + (n16 >> 2)) * FROW + (wave * 128 + 4 * (n16 & 3)) * 2;
     auto tr_read = [&](int mb) {
+      if (SCORES) return;
       tr[2 * mb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4f*)(vt + mb * 32));
       tr[2 * mb + 1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4f*)(vt + mb * 32 + 4 * FROW));
     };
@@ -378,7 +397,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       wait_vmcnt<8>();      // this wave's rows of tile i+1 have landed (the 8 loads of tile i+2 may be in flight)
     } else {
       wait_vmcnt<0>();
-      if (sm_valid && n16 == 0) { ml_lds[2 * sm_head] = m_ref; ml_lds[2 * sm_head + 1] = l_run; }   // final state for the epilogue
+      if (!SCORES && sm_valid && n16 == 0) { ml_lds[2 * sm_head] = m_ref; ml_lds[2 * sm_head + 1] = l_run; }   // final state for the epilogue
     }
     __syncthreads();        // B_c: P and rescale factors of tile i-1 are visible; tile i+1 is complete for every wave;
                             // the transposed reads of tile i-1 have returned, so its ring slot is free
@@ -387,10 +406,11 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     vec8 at_next[6], qop_next[4];
     const T* qrow = qhat + (i & 1) * (8 * 128) + (n32 < G ? n32 : G - 1) * 128 + (dq * 2 + g2) * 8;
     auto pv_step = [&](int mb) {
+      if (SCORES) return;
       vec8 a = __builtin_bit_cast(vec8, (s16x8f)__builtin_shufflevector(tr[2 * mb], tr[2 * mb + 1], 0, 1, 2, 3, 4, 5, 6, 7));
       acc[mb] = Elem<T>::mfma16(a, pb, acc[mb]);
     };
-    if (DO_PREV) {
+    if (DO_PREV && !SCORES) {
       const float al = alpha_lds[n16];
       pb = ld16<vec8>(p_lds + n16 * FP_ROW + 8 * g4);
       if (__builtin_amdgcn_ballot_w64(al != 1.f)) {   // rare: the softmax reference moved
@@ -455,6 +475,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   if (ntiles & 1) iteration(ntiles, IC<1>(), IC<0>(), IC<1>(), IC<0>());
   else iteration(ntiles, IC<0>(), IC<0>(), IC<1>(), IC<0>());
   __syncthreads();
+  if (SCORES) return;
 
   // ---- epilogue ----------------------------------------------------------------------------------------------------------
   if (n16 < G) {
@@ -474,7 +495,7 @@ template <typename T>
 int launch_recon_fast_t(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, hipStream_t st) {
   const int nb = sBb == 0 ? 1 : batch;   // one packed copy when the factor is shared by the batch
   pack_b_kernel<T><<<dim3(p.hkv, nb, 32), dim3(256), 0, st>>>((const T*)kB, (T*)p.Bp, sBb, sBh, sBr, p.hkv);
-  auto kern = recon_fast_kernel<T>;
+  auto kern = p.scores ? recon_fast_kernel<T, true> : recon_fast_kernel<T, false>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)FAST_SHM);
   if (e != hipSuccess) return (int)e;

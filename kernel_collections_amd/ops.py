@@ -147,7 +147,7 @@ def recon_stage1(q3, kA, kB, vA, partial, lse, scores, num_kv_splits, kv_lens, b
                  sm_scale, rope, inv_freq, pos_offset, sin_cos):
     a_op = kv_operand(kA, kA.stride(0), kA.stride(1), 0, kA.shape[-1])
     ws, ws_bytes = None, 0
-    if scores is None and USE_RECON_WORKSPACE:
+    if USE_RECON_WORKSPACE:
         ws_bytes = _lib.lib().xkv_recon_workspace_bytes(batch, hkv, kA.shape[-1], c_int64(kB.stride(0)))
         if ws_bytes:
             ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=q3.device)
