@@ -95,3 +95,13 @@ def test_random_mla(dev, H, L, dtype):
     scale = 1 / math.sqrt(192)
     out = mla2.mla_decode_attention_fwd(*(t.to(dev) for t in (qn, qr, ckv, kpe)), scale)
     check_out(out, oracle.mla_ref(*f32(qn, qr, ckv, kpe), scale), "mla")
+
+
+def test_profiling_cli_runs_and_agrees(dev, capsys):
+    """The variant table of kernel_collections_amd.profiling at a small shape: every non-RoPE row answers the same question
+    as eager attention."""
+    from kernel_collections_amd import profiling
+    rows = profiling.main(["--kv_len", "2048", "--k_rank", "256", "--v_rank", "512", "--batch", "2", "--warmup", "1", "--repeat", "2"])
+    assert len(rows) == 8 and "Fused xKV v2" in capsys.readouterr().out
+    for name, t, err in rows:
+        assert t > 0 and (math.isnan(err) or err < 3e-2), (name, err)
