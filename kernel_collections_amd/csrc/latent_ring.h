@@ -17,7 +17,8 @@ struct LatentParams {
 };
 typedef LatentParams RingParams;
 
-// True when the shape is one the ring kernel is built for (512-wide latent rows, optionally + 64 RoPE features, V the
+// True when the shape is one the ring kernel is built for (512-wide latent rows - or 384 / 256 with an absorbed query -
+// optionally + 64 RoPE features, V the
 // latent itself or scores-only; or two row streams: keys 512 / 1024 wide, values 512 wide); everything else runs the
 // register-staged kernel.
 bool ring_eligible(const RingParams& p, bool vshared);

@@ -1,4 +1,4 @@
-// Split-K flash-decoding stage 1 for WIDE latent rows (512 or 1024 features, optionally + 64 RoPE features):
+// Split-K flash-decoding stage 1 for WIDE latent rows (256 .. 1024 features, optionally + 64 RoPE features):
 // the bandwidth-bound scans of the path (absorbed no-PE xKV scores and decode, MLA over c_kv | k_pe, V-only
 // factorised decode with the per-head keys viewed as one 1024-wide row against a block-diagonal query).
 //
@@ -80,7 +80,8 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   constexpr int KS_W = NKS / KSPLIT;              // k-steps per wave
   static_assert(NKS % KSPLIT == 0, "the k-ranges are equal");
   static_assert(!HAS_R || TN == 32, "RoPE-key rows need 32-token tiles");
-  constexpr int IPR = DN / 512;                   // 1 KiB load instructions per C row
+  constexpr int IPR = DN > 512 ? DN / 512 : 1;    // load instructions per C row (1 KiB each; rows under 1 KiB use DN/8 lanes)
+  constexpr bool CPART = DN < 512;               // a C row fills only part of a load instruction
   // who issues the tile loads: the four compute waves (NLOAD == 0) or NLOAD extra waves that do nothing else, so that a
   // load instruction stalled on a full memory queue never holds up the MFMA / softmax work
   constexpr int NISS = NLOAD ? NLOAD : 4;
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   constexpr int RIW = 4 / NISS;                   // RoPE-key load instructions per issuing wave (4 per tile)
   constexpr int LPT = RPW * IPR + (HAS_R ? RIW : 0) + (VMODE == RING_VDISTINCT ? RPW : 0);   // loads per issuing wave per tile
   constexpr int WAITN = (RSLOT - 2) * LPT < 63 ? (RSLOT - 2) * LPT : 63;   // vmcnt holds 6 bits
-  constexpr int DV = 512, NVB = DV / 64;          // value features, 16-feature blocks per wave
+  constexpr int DV = VMODE == RING_VSHARED ? DN : 512, NVB = DV / 64;   // value features, 16-feature blocks per wave
   constexpr int TPH = 256 / HB, TPT = TN / TPH;   // softmax threads per head row, tokens per thread
   static_assert(TPT >= 1, "tile too short for the softmax thread map");
 
@@ -137,7 +138,8 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
 #pragma unroll
       for (int r = 0; r < RPW; ++r) {
 #pragma unroll
-        for (int c = 0; c < IPR; ++c) ring_load16(row + c * 1024, lane_off, slot + (iw * RPW + r) * CROW + c * 1024);
+        for (int c = 0; c < IPR; ++c)
+          if (!CPART || lane < DN / 8) ring_load16(row + c * 1024, lane_off, slot + (iw * RPW + r) * CROW + c * 1024);
         row += crow_bytes;
       }
       if (VMODE == RING_VDISTINCT) {
@@ -155,7 +157,8 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
         tok = tok < last ? tok : last;   // rows past the split end are masked in the softmax; keep the read in bounds
         const unsigned char* row = Cb + (int64_t)tok * crow_bytes;
 #pragma unroll
-        for (int c = 0; c < IPR; ++c) ring_load16(row + c * 1024, lane_off, slot + (iw * RPW + r) * CROW + c * 1024);
+        for (int c = 0; c < IPR; ++c)
+          if (!CPART || lane < DN / 8) ring_load16(row + c * 1024, lane_off, slot + (iw * RPW + r) * CROW + c * 1024);
         if (VMODE == RING_VDISTINCT)
           ring_load16(Vb + (int64_t)tok * vrow_bytes, lane_off, slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW);
       }
@@ -398,7 +401,7 @@ static int launch_ring_t(const RingParams& p, int batch, hipStream_t st) {
 // which instantiation serves a call; -1: none (the register-staged kernel runs instead)
 static int ring_vmode(const RingParams& p, bool vshared) {
   if (p.scores) return RING_SCORES;
-  if (vshared && p.dn == 512 && p.dv == 512) return RING_VSHARED;
+  if (vshared && p.dv == p.dn && (p.dn == 512 || p.dn == 384 || p.dn == 256)) return RING_VSHARED;
   if (!vshared && p.dv == 512) return RING_VDISTINCT;
   return -1;
 }
@@ -420,6 +423,13 @@ static int launch_ring_dt(const RingParams& p, int batch, bool vshared, hipStrea
   XKV_RING_CASE(16, 1, false, 512, false, RING_VDISTINCT)  XKV_RING_CASE(16, 2, false, 512, false, RING_VDISTINCT)
   XKV_RING_CASE(16, 1, true, 512, false, RING_VDISTINCT)   XKV_RING_CASE(16, 2, true, 512, false, RING_VDISTINCT)
   XKV_RING_CASE(16, 1, false, 1024, false, RING_VDISTINCT) XKV_RING_CASE(16, 2, false, 1024, false, RING_VDISTINCT)
+  // ranks 384 and 256 (absorbed queries always carry a low part)
+  XKV_RING_CASE(32, 1, true, 384, false, RING_SCORES)    XKV_RING_CASE(32, 2, true, 384, false, RING_SCORES)
+  XKV_RING_CASE(32, 1, true, 384, false, RING_VSHARED)   XKV_RING_CASE(32, 2, true, 384, false, RING_VSHARED)
+  XKV_RING_CASE(16, 1, true, 384, false, RING_VDISTINCT) XKV_RING_CASE(16, 2, true, 384, false, RING_VDISTINCT)
+  XKV_RING_CASE(32, 1, true, 256, false, RING_SCORES)    XKV_RING_CASE(32, 2, true, 256, false, RING_SCORES)
+  XKV_RING_CASE(32, 1, true, 256, false, RING_VSHARED)   XKV_RING_CASE(32, 2, true, 256, false, RING_VSHARED)
+  XKV_RING_CASE(16, 1, true, 256, false, RING_VDISTINCT) XKV_RING_CASE(16, 2, true, 256, false, RING_VDISTINCT)
 #undef XKV_RING_CASE
   return XKV_EUNSUPPORTED;
 }
@@ -428,7 +438,7 @@ bool ring_eligible(const RingParams& p, bool vshared) {
   const int hg = p.hq / p.groups, vm = ring_vmode(p, vshared);
   const bool lo = p.qn_lo != nullptr, r = p.R != nullptr;
   if (hg > 32 || vm < 0) return false;
-  if (p.dn != 512 && !(p.dn == 1024 && vm == RING_VDISTINCT && !lo)) return false;
+  if (p.dn != 512 && !(p.dn == 1024 && vm == RING_VDISTINCT && !lo) && !((p.dn == 384 || p.dn == 256) && lo && !r)) return false;
   if (r && (p.dr != 64 || lo || vm != RING_VSHARED)) return false;
   if (p.sCl < p.dn || (r && p.sRl < 64) || (vm == RING_VDISTINCT && p.sVl < 512)) return false;
   // the RoPE-key load addresses rows with a 32-bit byte offset from the sequence's first row

@@ -84,7 +84,7 @@ def mla_decode_attention_fwd_pd_sep_xKV(q, k_A_buffer, k_B_buffer, v_A_buffer, v
 
     # prefix: q absorbed into k_B (the reference's torch.matmul at :178), scan over k_A / v_A, partials in rank space
     qt_hi, qt_lo = ops.absorb_q(q3, k_B_buffer, want_lo=True)
-    S1 = ops.latent_splits(batch, groups, prefill_kv_len, rank)
+    S1 = ops.latent_splits(batch, groups, prefill_kv_len, rank, absorbed=True)
     splits1 = ops.uniform_splits(batch, S1, q.device)
     part1, lse1 = ops.workspaces(batch, num_q_heads, S1, rank_v, q.device)
     shared = v_A.data_ptr() == k_A.data_ptr() and v_A.stride() == k_A.stride() and rank_v == rank

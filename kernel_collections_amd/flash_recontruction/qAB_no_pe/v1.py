@@ -42,7 +42,7 @@ def qAB(q: torch.Tensor, Ak: torch.Tensor, Bk: torch.Tensor, *,
     qt_hi, qt_lo = ops.absorb_q(q3, Bk, want_lo=True)
     out = torch.empty((bsz, num_heads, 1, kv_len), dtype=out_dtype, device=q.device)
     groups = ops.head_groups(num_heads)
-    n_splits = ops.latent_splits(bsz, groups, kv_len, rank)
+    n_splits = ops.latent_splits(bsz, groups, kv_len, rank, absorbed=True)
     splits = ops.uniform_splits(bsz, n_splits, q.device)
     ops.latent_stage1(qt_hi, qt_lo, None, (Ak, Ak.stride(0), Ak.stride(1), 0, rank), None, None,
                       None, None, out, splits, None, bsz, num_heads, groups, kv_len, n_splits,

@@ -72,10 +72,11 @@ def settled_splits(kv_len: int, n: int) -> int:
         n = live
 
 
-def latent_splits(batch: int, groups: int, kv_len: int, width: int) -> int:
-    """Split count for the dot-product stage 1: 512-wide rows run the LDS-ring kernel (one workgroup per CU,
-    32-token tiles), everything else the register-staged one (two workgroups per CU, 64-token tiles)."""
-    if width == 512:
+def latent_splits(batch: int, groups: int, kv_len: int, width: int, absorbed: bool = False) -> int:
+    """Split count for the dot-product stage 1.  512-wide rows - and 256- / 384-wide ones scanned with an absorbed
+    query (hi + lo parts, no RoPE features) - run the LDS-ring kernel (one workgroup per CU, 32-token tiles);
+    everything else the register-staged one (two workgroups per CU, 64-token tiles)."""
+    if width == 512 or (absorbed and width in (256, 384)):
         return occupancy_splits(batch, groups, kv_len, tile=32, waves=1)
     return occupancy_splits(batch, groups, kv_len)
 

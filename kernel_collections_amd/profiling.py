@@ -62,7 +62,7 @@ def build_variants(batch, hq, hkv, d, L, rk, rv, dtype, dev, theta=5e5):
     scale = 1.0 / math.sqrt(d)
     S = ops.occupancy_splits(batch, hkv, L)
     ns = ops.uniform_splits(batch, S, dev)
-    S1 = ops.latent_splits(batch, 1, L, rk)
+    S1 = ops.latent_splits(batch, 1, L, rk, absorbed=True)
     ns1 = ops.uniform_splits(batch, S1, dev)
     Sr = ops.occupancy_splits(batch, hkv, L, tile=32, waves=1)
     Sv = ops.occupancy_splits(batch, 1, L, tile=32, waves=1)   # V-only factorised: one workgroup serves every head of a split
