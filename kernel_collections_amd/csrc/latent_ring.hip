@@ -48,13 +48,13 @@ __device__ __forceinline__ f32x4 mfma16k16(_Float16, s16x4r a, s16x4r b, f32x4 c
 
 enum { RING_SCORES = 0, RING_VSHARED = 1, RING_VDISTINCT = 2 };
 
-template <int TN, int DN, bool HAS_R, int VMODE, int NHB>
+template <int TN, int DN, bool HAS_R, int VMODE, int NHB, int DVW>
 struct RingShape {
   static constexpr int HB = 16 * NHB;
   static constexpr int CROW = DN * 2 + 16;                 // padded C row (bytes)
   static constexpr int CBYTES = TN * CROW;
   static constexpr int RBYTES = HAS_R ? TN * 128 : 0;
-  static constexpr int VROW = 512 * 2 + 16;                // padded V row (distinct-V mode)
+  static constexpr int VROW = DVW * 2 + 16;                // padded V row (distinct-V mode)
   static constexpr int VBYTES = VMODE == RING_VDISTINCT ? TN * VROW : 0;
   static constexpr int SLOT = CBYTES + RBYTES + VBYTES;
   static constexpr int KSPLIT = 4 / (TN / 16);             // k-ranges (waves per 16-token block)
@@ -68,11 +68,11 @@ struct RingShape {
 
 // T: operand type; TN: tokens per tile (32, or 16 when two row streams share the LDS); NHB: 16-row head blocks; LO: q has
 // a low-order part; DN: latent width; HAS_R: 64 RoPE features follow (TN 32 only); VMODE: scores only / V is the first
-// 512 features of the C row / V is a second 512-wide row stream.
-template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE, int NLOAD>
+// DN features of the C row / V is a second, DVW-wide row stream.
+template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE, int DVW, int NLOAD>
 __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const RingParams p) {
   typedef typename Elem<T>::vec8 vec8;
-  typedef RingShape<TN, DN, HAS_R, VMODE, NHB> S;
+  typedef RingShape<TN, DN, HAS_R, VMODE, NHB, DVW> S;
   constexpr bool SCORES = VMODE == RING_SCORES;
   constexpr int HB = S::HB, CROW = S::CROW, CBYTES = S::CBYTES, VROW = S::VROW, SLOT = S::SLOT, RSLOT = S::RSLOT;
   constexpr int NTB = TN / 16, KSPLIT = S::KSPLIT, SP = S::SP, LDP = S::LDP;
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   constexpr int RIW = 4 / NISS;                   // RoPE-key load instructions per issuing wave (4 per tile)
   constexpr int LPT = RPW * IPR + (HAS_R ? RIW : 0) + (VMODE == RING_VDISTINCT ? RPW : 0);   // loads per issuing wave per tile
   constexpr int WAITN = (RSLOT - 2) * LPT < 63 ? (RSLOT - 2) * LPT : 63;   // vmcnt holds 6 bits
-  constexpr int DV = VMODE == RING_VSHARED ? DN : 512, NVB = DV / 64;   // value features, 16-feature blocks per wave
+  constexpr int DV = VMODE == RING_VSHARED ? DN : DVW, NVB = DV / 64;   // value features, 16-feature blocks per wave
   constexpr int TPH = 256 / HB, TPT = TN / TPH;   // softmax threads per head row, tokens per thread
   static_assert(TPT >= 1, "tile too short for the softmax thread map");
 
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
         const unsigned char* vrow = Vb + (int64_t)tok0 * vrow_bytes;
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
-          ring_load16(vrow, lane_off, slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW);
+          if (DVW >= 512 || lane < DVW / 8) ring_load16(vrow, lane_off, slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW);
           vrow += vrow_bytes;
         }
       }
@@ -160,7 +160,8 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
         for (int c = 0; c < IPR; ++c)
           if (!CPART || lane < DN / 8) ring_load16(row + c * 1024, lane_off, slot + (iw * RPW + r) * CROW + c * 1024);
         if (VMODE == RING_VDISTINCT)
-          ring_load16(Vb + (int64_t)tok * vrow_bytes, lane_off, slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW);
+          if (DVW >= 512 || lane < DVW / 8)
+            ring_load16(Vb + (int64_t)tok * vrow_bytes, lane_off, slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW);
       }
     }
     if (HAS_R) {
@@ -386,11 +387,11 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
 #ifndef XKV_RING_NLOAD
 #define XKV_RING_NLOAD 2
 #endif
-template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE>
+template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE, int DVW = 512>
 static int launch_ring_t(const RingParams& p, int batch, hipStream_t st) {
-  constexpr int SHM = RingShape<TN, DN, HAS_R, VMODE, NHB>::SHM;
+  constexpr int SHM = RingShape<TN, DN, HAS_R, VMODE, NHB, DVW>::SHM;
   constexpr int NLOAD = XKV_RING_NLOAD;
-  auto kern = latent_ring_kernel<T, TN, NHB, LO, DN, HAS_R, VMODE, NLOAD>;
+  auto kern = latent_ring_kernel<T, TN, NHB, LO, DN, HAS_R, VMODE, DVW, NLOAD>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SHM);
   if (e != hipSuccess) return (int)e;
   const int total = batch * p.groups * p.max_splits;
@@ -402,7 +403,7 @@ static int launch_ring_t(const RingParams& p, int batch, hipStream_t st) {
 static int ring_vmode(const RingParams& p, bool vshared) {
   if (p.scores) return RING_SCORES;
   if (vshared && p.dv == p.dn && (p.dn == 512 || p.dn == 384 || p.dn == 256)) return RING_VSHARED;
-  if (!vshared && p.dv == 512) return RING_VDISTINCT;
+  if (!vshared && (p.dv == 512 || p.dv == 384 || p.dv == 256)) return RING_VDISTINCT;
   return -1;
 }
 
@@ -419,17 +420,23 @@ static int launch_ring_dt(const RingParams& p, int batch, bool vshared, hipStrea
   XKV_RING_CASE(32, 1, false, 512, false, RING_VSHARED)  XKV_RING_CASE(32, 2, false, 512, false, RING_VSHARED)
   XKV_RING_CASE(32, 1, true, 512, false, RING_VSHARED)   XKV_RING_CASE(32, 2, true, 512, false, RING_VSHARED)
   XKV_RING_CASE(32, 1, false, 512, true, RING_VSHARED)   XKV_RING_CASE(32, 2, false, 512, true, RING_VSHARED)
-  // two row streams (keys 512 or 1024 wide, values 512 wide): 16-token tiles
-  XKV_RING_CASE(16, 1, false, 512, false, RING_VDISTINCT)  XKV_RING_CASE(16, 2, false, 512, false, RING_VDISTINCT)
-  XKV_RING_CASE(16, 1, true, 512, false, RING_VDISTINCT)   XKV_RING_CASE(16, 2, true, 512, false, RING_VDISTINCT)
-  XKV_RING_CASE(16, 1, false, 1024, false, RING_VDISTINCT) XKV_RING_CASE(16, 2, false, 1024, false, RING_VDISTINCT)
-  // ranks 384 and 256 (absorbed queries always carry a low part)
+  // two row streams (keys 256 .. 1024 wide, values 256 .. 512 wide): 16-token tiles
+#define XKV_RING_V2(NHB, LO, DN, DVW) \
+  if (nhb == NHB && lo == LO && p.dn == DN && !r && vm == RING_VDISTINCT && p.dv == DVW) \
+    return launch_ring_t<T, 16, NHB, LO, DN, false, RING_VDISTINCT, DVW>(p, batch, st);
+#define XKV_RING_V2_ALL(LO, DN) \
+  XKV_RING_V2(1, LO, DN, 512) XKV_RING_V2(2, LO, DN, 512) XKV_RING_V2(1, LO, DN, 384) XKV_RING_V2(2, LO, DN, 384) \
+  XKV_RING_V2(1, LO, DN, 256) XKV_RING_V2(2, LO, DN, 256)
+  XKV_RING_V2_ALL(true, 512) XKV_RING_V2_ALL(true, 384) XKV_RING_V2_ALL(true, 256)   // absorbed query, both factorised
+  XKV_RING_V2_ALL(false, 1024)                                                       // per-head keys as one row, V factorised
+  XKV_RING_V2(1, false, 512, 512) XKV_RING_V2(2, false, 512, 512)                    // plain 512-wide keys and values
+#undef XKV_RING_V2_ALL
+#undef XKV_RING_V2
+  // ranks 384 and 256, one stream (absorbed queries always carry a low part)
   XKV_RING_CASE(32, 1, true, 384, false, RING_SCORES)    XKV_RING_CASE(32, 2, true, 384, false, RING_SCORES)
   XKV_RING_CASE(32, 1, true, 384, false, RING_VSHARED)   XKV_RING_CASE(32, 2, true, 384, false, RING_VSHARED)
-  XKV_RING_CASE(16, 1, true, 384, false, RING_VDISTINCT) XKV_RING_CASE(16, 2, true, 384, false, RING_VDISTINCT)
   XKV_RING_CASE(32, 1, true, 256, false, RING_SCORES)    XKV_RING_CASE(32, 2, true, 256, false, RING_SCORES)
   XKV_RING_CASE(32, 1, true, 256, false, RING_VSHARED)   XKV_RING_CASE(32, 2, true, 256, false, RING_VSHARED)
-  XKV_RING_CASE(16, 1, true, 256, false, RING_VDISTINCT) XKV_RING_CASE(16, 2, true, 256, false, RING_VDISTINCT)
 #undef XKV_RING_CASE
   return XKV_EUNSUPPORTED;
 }
@@ -440,7 +447,8 @@ bool ring_eligible(const RingParams& p, bool vshared) {
   if (hg > 32 || vm < 0) return false;
   if (p.dn != 512 && !(p.dn == 1024 && vm == RING_VDISTINCT && !lo) && !((p.dn == 384 || p.dn == 256) && lo && !r)) return false;
   if (r && (p.dr != 64 || lo || vm != RING_VSHARED)) return false;
-  if (p.sCl < p.dn || (r && p.sRl < 64) || (vm == RING_VDISTINCT && p.sVl < 512)) return false;
+  if (p.sCl < p.dn || (r && p.sRl < 64) || (vm == RING_VDISTINCT && p.sVl < p.dv)) return false;
+  if (vm == RING_VDISTINCT && p.dn == 512 && !lo && p.dv != 512) return false;
   // the RoPE-key load addresses rows with a 32-bit byte offset from the sequence's first row
   if (r && (int64_t)p.kv_len * p.sRl * 2 >= (int64_t)1 << 31) return false;
   return true;

@@ -58,7 +58,8 @@ def decode_attention_fwd_v_factorized(q, k_buffer, v_A_buffer, v_B_buffer, o, nu
     q3 = ops._q3(q)
     k_buffer, v_A_buffer = ops.as_rows(k_buffer), ops.as_rows(v_A_buffer)
     partial, lse = ops.workspaces(batch, hq, S, rv, q.device)
-    if hkv * d in (512, 1024) and rv == 512 and hq <= 32 and k_buffer.stride(2) == d:
+    wide = (hkv * d == 1024 and rv in (256, 384, 512)) or (hkv * d == 512 and rv == 512)
+    if wide and hq <= 32 and k_buffer.stride(2) == d:
         # all heads from one workgroup: the token's keys are one hkv*d-wide row against a block-diagonal query, and the
         # value basis (shared by the heads) is read once per token instead of once per kv head
         qbd = ops.blockdiag_q(q3, hkv)
