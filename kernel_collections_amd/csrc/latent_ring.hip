@@ -46,7 +46,8 @@ __device__ __forceinline__ f32x4 mfma16k16(_Float16, s16x4r a, s16x4r b, f32x4 c
   return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4r, a), __builtin_bit_cast(f16x4r, b), c, 0, 0, 0);
 }
 
-enum { RING_SCORES = 0, RING_VSHARED = 1, RING_VDISTINCT = 2 };
+enum { RING_SCORES = 0, RING_VSHARED = 1, RING_VDISTINCT = 2, RING_VHEADS = 3 };
+constexpr int RING_DVH = 128;   // head width of the per-head value rows (RING_VHEADS)
 
 template <int TN, int DN, bool HAS_R, int VMODE, int NHB, int DVW>
 struct RingShape {
@@ -55,7 +56,7 @@ struct RingShape {
   static constexpr int CBYTES = TN * CROW;
   static constexpr int RBYTES = HAS_R ? TN * 128 : 0;
   static constexpr int VROW = DVW * 2 + 16;                // padded V row (distinct-V mode)
-  static constexpr int VBYTES = VMODE == RING_VDISTINCT ? TN * VROW : 0;
+  static constexpr int VBYTES = VMODE >= RING_VDISTINCT ? TN * VROW : 0;
   static constexpr int SLOT = CBYTES + RBYTES + VBYTES;
   static constexpr int KSPLIT = 4 / (TN / 16);             // k-ranges (waves per 16-token block)
   static constexpr int SP = TN + 4;                        // partial-score row stride (floats)
@@ -68,12 +69,16 @@ struct RingShape {
 
 // T: operand type; TN: tokens per tile (32, or 16 when two row streams share the LDS); NHB: 16-row head blocks; LO: q has
 // a low-order part; DN: latent width; HAS_R: 64 RoPE features follow (TN 32 only); VMODE: scores only / V is the first
-// DN features of the C row / V is a second, DVW-wide row stream.
+// DN features of the C row / V is a second, DVW-wide row stream / V is a second stream of DVW / 128 per-kv-head value
+// rows of 128 features (plain values under absorbed factorised keys): the workgroup serves every query head, wave w
+// accumulates kv heads 2w, 2w+1, and query head h multiplies the values of kv head h / (heads per kv head).
 template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE, int DVW, int NLOAD>
 __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const RingParams p) {
   typedef typename Elem<T>::vec8 vec8;
   typedef RingShape<TN, DN, HAS_R, VMODE, NHB, DVW> S;
-  constexpr bool SCORES = VMODE == RING_SCORES;
+  constexpr bool SCORES = VMODE == RING_SCORES, V2 = VMODE >= RING_VDISTINCT, VHEADS = VMODE == RING_VHEADS;
+  constexpr int VIPR = DVW > 512 ? DVW / 512 : 1;   // load instructions per V row
+  constexpr int KVH = DVW / RING_DVH, KVW = VHEADS ? KVH / 4 : 1;   // kv heads of a value row, per wave
   constexpr int HB = S::HB, CROW = S::CROW, CBYTES = S::CBYTES, VROW = S::VROW, SLOT = S::SLOT, RSLOT = S::RSLOT;
   constexpr int NTB = TN / 16, KSPLIT = S::KSPLIT, SP = S::SP, LDP = S::LDP;
   constexpr int NKS_N = DN / 32, NKS = NKS_N + (HAS_R ? 2 : 0);
@@ -87,9 +92,12 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   constexpr int NISS = NLOAD ? NLOAD : 4;
   constexpr int RPW = TN / NISS;                  // rows per issuing wave per tile
   constexpr int RIW = 4 / NISS;                   // RoPE-key load instructions per issuing wave (4 per tile)
-  constexpr int LPT = RPW * IPR + (HAS_R ? RIW : 0) + (VMODE == RING_VDISTINCT ? RPW : 0);   // loads per issuing wave per tile
+  constexpr int LPT = RPW * IPR + (HAS_R ? RIW : 0) + (V2 ? RPW * VIPR : 0);   // loads per issuing wave per tile
   constexpr int WAITN = (RSLOT - 2) * LPT < 63 ? (RSLOT - 2) * LPT : 63;   // vmcnt holds 6 bits
-  constexpr int DV = VMODE == RING_VSHARED ? DN : DVW, NVB = DV / 64;   // value features, 16-feature blocks per wave
+  constexpr int DV = VMODE == RING_VSHARED ? DN : VHEADS ? RING_DVH : DVW;   // value features of an output row
+  constexpr int NVB = VHEADS ? RING_DVH / 16 : DV / 64;   // 16-feature blocks per wave (per kv head under VHEADS)
+  constexpr int NA2 = VHEADS ? KVW : NHB;
+  static_assert(!VHEADS || (TN == 16 && KVH % 4 == 0), "per-head values: 16-token tiles, kv heads split over 4 waves");
   constexpr int TPH = 256 / HB, TPT = TN / TPH;   // softmax threads per head row, tokens per thread
   static_assert(TPT >= 1, "tile too short for the softmax thread map");
 
@@ -125,7 +133,7 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   const unsigned char* Cb = reinterpret_cast<const unsigned char*>(p.C) + (b * p.sCb + group * p.sCh) * 2;
   const unsigned char* Rb = HAS_R ? reinterpret_cast<const unsigned char*>(p.R) + (b * p.sRb + group * p.sRh) * 2 : nullptr;
   const unsigned char* Vb =
-      VMODE == RING_VDISTINCT ? reinterpret_cast<const unsigned char*>(p.V) + (b * p.sVb + group * p.sVh) * 2 : nullptr;
+      V2 ? reinterpret_cast<const unsigned char*>(p.V) + (b * p.sVb + (VHEADS ? 0 : group * p.sVh)) * 2 : nullptr;
   const int64_t crow_bytes = p.sCl * 2, rrow_bytes = p.sRl * 2, vrow_bytes = p.sVl * 2;
   const unsigned lane_off = lane * 16;
   const int r_row = lane & 31;
@@ -142,11 +150,14 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
           if (!CPART || lane < DN / 8) ring_load16(row + c * 1024, lane_off, slot + (iw * RPW + r) * CROW + c * 1024);
         row += crow_bytes;
       }
-      if (VMODE == RING_VDISTINCT) {
+      if (V2) {
         const unsigned char* vrow = Vb + (int64_t)tok0 * vrow_bytes;
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
-          if (DVW >= 512 || lane < DVW / 8) ring_load16(vrow, lane_off, slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW);
+#pragma unroll
+          for (int c = 0; c < VIPR; ++c)
+            if (DVW >= 512 || lane < DVW / 8)
+              ring_load16(vrow + c * 1024, lane_off, slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW + c * 1024);
           vrow += vrow_bytes;
         }
       }
@@ -159,9 +170,13 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
 #pragma unroll
         for (int c = 0; c < IPR; ++c)
           if (!CPART || lane < DN / 8) ring_load16(row + c * 1024, lane_off, slot + (iw * RPW + r) * CROW + c * 1024);
-        if (VMODE == RING_VDISTINCT)
-          if (DVW >= 512 || lane < DVW / 8)
-            ring_load16(Vb + (int64_t)tok * vrow_bytes, lane_off, slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW);
+        if (V2) {
+#pragma unroll
+          for (int c = 0; c < VIPR; ++c)
+            if (DVW >= 512 || lane < DVW / 8)
+              ring_load16(Vb + (int64_t)tok * vrow_bytes + c * 1024, lane_off,
+                          slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW + c * 1024);
+        }
       }
     }
     if (HAS_R) {
@@ -227,11 +242,12 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   // ---- running state ---------------------------------------------------------------------------------------------
   const int srow = tid / TPH, ssub = tid % TPH;
   float m_run = NEG_INF, l_run = 0.f;
-  f32x4 acc[SCORES ? 1 : NVB][NHB];
+  f32x4 acc[SCORES ? 1 : NVB][NA2];
 #pragma unroll
   for (int mb = 0; mb < (SCORES ? 1 : NVB); ++mb)
 #pragma unroll
-    for (int hb = 0; hb < NHB; ++hb) acc[mb][hb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int hb = 0; hb < NA2; ++hb) acc[mb][hb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int hpk = VHEADS ? hg / KVH : 0;   // query heads per kv head
   const int vcol0 = wave * (DV / 4);
 
   for (int t = 0; t < ntiles; ++t) {
@@ -331,7 +347,22 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
     __syncthreads();                  // C: P and alpha of tile t are visible
 
     // ---- PV: acc^T[feature, head] += V^T P^T, this wave's quarter of the value features -----------------------------
-    {
+    if (VHEADS) {
+      // per kv head j of this wave: acc^T[feature, query head of j] += V_j^T P^T; column n16 of the P operand is query
+      // head hpk * j + n16 (columns past the heads of j repeat the last row and are never written out)
+      const unsigned char* vbase = slot + CBYTES + S::RBYTES;
+#pragma unroll
+      for (int j = 0; j < KVW; ++j) {
+        const int kvh = wave * KVW + j;
+        int prow = hpk * kvh + n16;
+        prow = prow < HB - 1 ? prow : HB - 1;
+        const float al = alpha_lds[prow];
+        const s16x4r pb = *reinterpret_cast<const s16x4r*>(p_lds + prow * LDP + 4 * g4);
+        const unsigned char* vrow = vbase + (4 * g4 + (n16 >> 2)) * VROW + (kvh * RING_DVH + 4 * (n16 & 3)) * 2;
+#pragma unroll
+        for (int mb = 0; mb < NVB; ++mb) acc[mb][j] = mfma16k16(T(), ring_tr4(vrow + mb * 32), pb, acc[mb][j] * al);
+      }
+    } else {
       constexpr int VR = VMODE == RING_VDISTINCT ? VROW : CROW;
       const unsigned char* vbase = slot + (VMODE == RING_VDISTINCT ? CBYTES + S::RBYTES : 0);
       float al[NHB];
@@ -369,6 +400,22 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   // ---- epilogue: normalise, write partial + lse --------------------------------------------------------------------
   if (ssub == 0) { ml_lds[2 * srow] = m_run; ml_lds[2 * srow + 1] = l_run; }
   __syncthreads();
+  if (VHEADS) {
+#pragma unroll
+    for (int j = 0; j < KVW; ++j) {
+      const int hrow = hpk * (wave * KVW + j) + n16;
+      if (n16 < hpk) {
+        const float m = ml_lds[2 * hrow], l = ml_lds[2 * hrow + 1];
+        const float inv = 1.f / l;
+        const int64_t ph = ((int64_t)b * p.hq + hrow) * p.max_splits + split;
+        float* dst = p.partial + ph * RING_DVH + 4 * g4;
+#pragma unroll
+        for (int mb = 0; mb < NVB; ++mb) *reinterpret_cast<f32x4*>(dst + mb * 16) = acc[mb][j] * inv;
+        if (g4 == 0) p.lse[ph] = m + __logf(l);
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int hb = 0; hb < NHB; ++hb) {
     const int hrow = hb * 16 + n16;
@@ -400,8 +447,17 @@ static int launch_ring_t(const RingParams& p, int batch, hipStream_t st) {
 }
 
 // which instantiation serves a call; -1: none (the register-staged kernel runs instead)
+// plain per-kv-head values [token][8 heads][128] under one shared, absorbed key basis: the call's kv groups all scan the
+// same C rows, so one workgroup per (sequence, split) serves every head
+static bool ring_vheads(const RingParams& p, bool vshared) {
+  return !p.scores && !vshared && p.groups * RING_DVH == 1024 && p.dv == RING_DVH && p.sVh == RING_DVH && p.sCh == 0 &&
+         p.qn_lo && !p.R && p.hq <= 32 && p.hq % p.groups == 0 && (p.dn == 512 || p.dn == 384 || p.dn == 256) &&
+         p.sCl >= p.dn && p.sVl >= 1024;
+}
+
 static int ring_vmode(const RingParams& p, bool vshared) {
   if (p.scores) return RING_SCORES;
+  if (ring_vheads(p, vshared)) return RING_VHEADS;
   if (vshared && p.dv == p.dn && (p.dn == 512 || p.dn == 384 || p.dn == 256)) return RING_VSHARED;
   if (!vshared && (p.dv == 512 || p.dv == 384 || p.dv == 256)) return RING_VDISTINCT;
   return -1;
@@ -411,6 +467,16 @@ template <typename T>
 static int launch_ring_dt(const RingParams& p, int batch, bool vshared, hipStream_t st) {
   const int hg = p.hq / p.groups, vm = ring_vmode(p, vshared);
   const bool lo = p.qn_lo != nullptr, r = p.R != nullptr;
+  if (vm == RING_VHEADS) {
+    RingParams a = p;
+    a.groups = 1;
+    a.total_wg = batch * p.max_splits;
+#define XKV_RING_VH(NHB, DN) \
+  if ((p.hq <= 16 ? 1 : 2) == NHB && p.dn == DN) return launch_ring_t<T, 16, NHB, true, DN, false, RING_VHEADS, 1024>(a, batch, st);
+    XKV_RING_VH(1, 512) XKV_RING_VH(2, 512) XKV_RING_VH(1, 384) XKV_RING_VH(2, 384) XKV_RING_VH(1, 256) XKV_RING_VH(2, 256)
+#undef XKV_RING_VH
+    return XKV_EUNSUPPORTED;
+  }
   const int nhb = hg <= 16 ? 1 : 2;
 #define XKV_RING_CASE(TN, NHB, LO, DN, HAS_R, VM) \
   if (nhb == NHB && lo == LO && p.dn == DN && r == HAS_R && vm == VM) return launch_ring_t<T, TN, NHB, LO, DN, HAS_R, VM>(p, batch, st);
@@ -444,6 +510,7 @@ static int launch_ring_dt(const RingParams& p, int batch, bool vshared, hipStrea
 bool ring_eligible(const RingParams& p, bool vshared) {
   const int hg = p.hq / p.groups, vm = ring_vmode(p, vshared);
   const bool lo = p.qn_lo != nullptr, r = p.R != nullptr;
+  if (vm == RING_VHEADS) return true;
   if (hg > 32 || vm < 0) return false;
   if (p.dn != 512 && !(p.dn == 1024 && vm == RING_VDISTINCT && !lo) && !((p.dn == 384 || p.dn == 256) && lo && !r)) return false;
   if (r && (p.dr != 64 || lo || vm != RING_VSHARED)) return false;
