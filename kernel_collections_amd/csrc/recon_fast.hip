@@ -258,11 +258,15 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     }
     s0 = tok < end ? s0 * p.sm_scale : NEG_INF;
     s1 = tok + 1 < end ? s1 * p.sm_scale : NEG_INF;
-    // the reference maximum only moves when the tile maximum exceeds it by LAZY_RESCALE (branch-free: alpha = 1 otherwise)
-    const float mx = row_reduce<true, 16>(fmaxf(s0, s1));
-    const float m_new = mx > m_ref + LAZY_RESCALE ? mx : m_ref;
-    const float alpha = __expf(m_ref - m_new);
-    m_ref = m_new;
+    // the reference maximum only moves when the tile maximum exceeds it by LAZY_RESCALE; the reduction that finds the
+    // maximum runs only then, so the usual path from scores to P has no cross-lane step
+    float alpha = 1.f;
+    if (__builtin_amdgcn_ballot_w64(fmaxf(s0, s1) > m_ref + LAZY_RESCALE)) {   // rare: some head's maximum moves
+      const float mx = row_reduce<true, 16>(fmaxf(s0, s1));
+      const float m_new = mx > m_ref + LAZY_RESCALE ? mx : m_ref;
+      alpha = __expf(m_ref - m_new);
+      m_ref = m_new;
+    }
     const float e0 = __expf(s0 - m_ref), e1 = __expf(s1 - m_ref);
     l_run = l_run * alpha + row_reduce<false, 16>(e0 + e1);
     T* pd = p_lds + sm_head * FP_ROW + 2 * n16;
