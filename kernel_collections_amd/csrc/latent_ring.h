@@ -17,10 +17,10 @@ struct LatentParams {
 };
 typedef LatentParams RingParams;
 
-// True when the shape is one the ring kernel is built for (512-wide latent rows - or 384 / 256 with an absorbed query -
-// optionally + 64 RoPE features, V the
-// latent itself or scores-only; or two row streams: keys 512 / 1024 wide, values 512 wide); everything else runs the
-// register-staged kernel.
+// True when the shape is one the ring kernel is built for: 512-wide latent rows (optionally + 64 RoPE features), or
+// 384 / 256 wide ones scanned with an absorbed query (hi + lo parts); V the latent itself, scores only, a second row
+// stream 256 / 384 / 512 wide (keys then 256 .. 1024 wide), or plain per-kv-head values [token][8][128] under one shared
+// absorbed key basis.  Everything else runs the register-staged kernel.
 bool ring_eligible(const RingParams& p, bool vshared);
 int launch_ring(const RingParams& p, int batch, bool vshared, int dtype, hipStream_t st);
 
