@@ -363,7 +363,7 @@ static int dispatch_recon(const ReconParams& p, int batch, bool vshared, hipStre
 using namespace xkv;
 
 extern "C" int64_t xkv_recon_workspace_bytes(int batch, int hkv, int rank, int64_t stride_kB_b) {
-  if (rank != 512) return 0;
+  if (rank != 512 && rank != 384 && rank != 256) return 0;
   return (int64_t)(stride_kB_b == 0 ? 1 : batch) * hkv * rank * 128 * 2;
 }
 
@@ -413,6 +413,24 @@ extern "C" int xkv_recon_stage1(const void* q_pe, xkv_kv_operand kA, const void*
     f.hq = hq; f.hkv = hkv; f.kv_len = kv_len; f.max_splits = max_splits; f.total_wg = batch * hkv * max_splits;
     f.sm_scale = sm_scale; f.inv_freq = inv_freq; f.pos_offset = pos_offset;
     return launch_recon_fast(f, kB, sBb, sBh, sBr, batch, dtype, st);
+  }
+  // 8-wave kernels: the other ranks, and a value basis of its own
+  if (rope && !sin_cos && hq / hkv <= 8 && workspace && need > 0 && workspace_bytes >= need &&
+      (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 && (int64_t)kA.stride_l * 2 * 3 < ((int64_t)1 << 31) &&
+      (so || vshared || (int64_t)vA.stride_l * 2 * 3 < ((int64_t)1 << 31))) {
+    FastParams f;
+    f.q = q_pe; f.kA = kA.ptr; f.Bp = workspace;
+    f.sAb = kA.stride_b; f.sAl = kA.stride_l; f.sBpb = sBb == 0 ? 0 : (int64_t)hkv * rank * 128;
+    f.partial = partial; f.lse = lse; f.scores = scores_out; f.scores_dtype = scores_dtype;
+    f.num_splits = num_kv_splits; f.kv_lens = kv_lens;
+    f.hq = hq; f.hkv = hkv; f.kv_len = kv_len; f.max_splits = max_splits; f.total_wg = batch * hkv * max_splits;
+    f.sm_scale = sm_scale; f.inv_freq = inv_freq; f.pos_offset = pos_offset;
+    f.vA = vA.ptr; f.sVb = vA.stride_b; f.sVl = vA.stride_l;
+    const int mode = so ? 0 : vshared ? 1 : 2, rv = so ? rank : vA.dim;
+    int rc = launch_recon_duo_a(f, kB, sBb, sBh, sBr, batch, dtype, mode, rank, rv, st);
+    if (rc == DUO_NOT_MINE) rc = launch_recon_duo_b(f, kB, sBb, sBh, sBr, batch, dtype, mode, rank, rv, st);
+    if (rc == DUO_NOT_MINE) rc = launch_recon_duo_c(f, kB, sBb, sBh, sBr, batch, dtype, mode, rank, rv, st);
+    if (rc != DUO_NOT_MINE) return rc;
   }
   return dtype == XKV_BF16 ? dispatch_recon<__bf16>(p, batch, vshared, st) : dispatch_recon<_Float16>(p, batch, vshared, st);
 }
