@@ -77,7 +77,8 @@ def test_qab_nope_shared_factor_stride0_and_row_strides(dev):
 # ------------------------------------------------------------------------------------ qAB with RoPE
 @pytest.mark.parametrize("dtype", [BF, FP])
 @pytest.mark.parametrize("b,hq,hkv,L,r,theta", [(2, 32, 8, 1000, 512, 5e5), (1, 8, 2, 77, 256, 1e7),
-                                                (1, 16, 1, 2085, 384, 1e4), (2, 4, 4, 40, 192, 1e7)])
+                                                (1, 16, 1, 2085, 384, 1e4), (2, 4, 4, 40, 192, 1e7),
+                                                (2, 8, 2, 300, 384, 5e5)])   # 8-wave kernel, scores mode
 def test_qab_rope(dev, dtype, b, hq, hkv, L, r, theta):
     d = 128
     q, A, B = gen((b, hq, 1, d), std=0.5, dtype=dtype, seed=1), gen((b, L, r), dtype=dtype, seed=2), \
@@ -173,6 +174,35 @@ def test_fused_rope(dev, dtype, b, hq, hkv, L, rk, rv, S, shared):
     o2 = torch.zeros_like(qd)
     fr.gqa_xKV_rope(qd, kAd, kBd, vAd, vBd, o2, splits_t([S] * b, dev), S, scale, sin_cos=table.to(dev))
     check_out(o2, ref_t, "gqa_xKV_rope table")
+
+
+@pytest.mark.parametrize("dtype", [BF, FP])
+@pytest.mark.parametrize("b,hq,hkv,rk,rv,shared,lens,S,off", [
+    (2, 32, 8, 512, 512, False, [1000, 333], 4, 0),        # every shape the 8-wave kernels are built for
+    (1, 16, 2, 384, 512, False, [2100], 3, 4096),          # 8 query heads per kv head
+    (2, 8, 8, 384, 384, False, [17, 64], 2, 0),            # shorter than a tile / exactly two tiles; one head per kv head
+    (3, 32, 8, 256, 256, False, [700, 5, 2048], 5, 100000),
+    (1, 24, 8, 256, 512, False, [1500], 7, 0),             # the last splits are dead
+    (2, 32, 8, 384, 384, True, [900, 1200], 4, 0),
+    (2, 16, 4, 256, 256, True, [33, 4000], 6, 131072 - 4000)])
+def test_fused_rope_wide_kernels(dev, dtype, b, hq, hkv, rk, rv, shared, lens, S, off):
+    d, theta = 128, 5e5
+    L = max(lens)
+    q = gen((b, hq, d), std=0.4, dtype=dtype, seed=21)
+    kA, kB = gen((b, L, rk), dtype=dtype, seed=22), gen((b, hkv, rk, d), std=rk ** -0.5, dtype=dtype, seed=23)
+    vA = kA if shared else gen((b, L, rv), dtype=dtype, seed=24)
+    vB = gen((b, hkv, vA.shape[-1], d), std=vA.shape[-1] ** -0.5, dtype=dtype, seed=25)
+    scale = d ** -0.5
+    qd, kAd, kBd, vBd = dev_(dev, q, kA, kB, vB)
+    vAd = kAd if shared else vA.to(dev)
+    o = torch.zeros_like(qd)
+    fr.gqa_xKV_rope(qd, kAd, kBd, vAd, vBd, o, splits_t([S] * b, dev), S, scale, theta, pos_offset=off,
+                    kv_lens=torch.tensor(lens, dtype=torch.int32, device=dev))
+    for i, n in enumerate(lens):   # every sequence against the oracle on its own length
+        cos, sin = oracle.rope_cos_sin(torch.arange(off, off + n), d, theta)
+        ref = oracle.gqa_factorized_rope(*f32(q[i:i + 1].unsqueeze(2), kA[i:i + 1, :n], kB[i:i + 1], vA[i:i + 1, :n], vB[i:i + 1]),
+                                         cos, sin, sm_scale=scale)[:, :, 0]
+        check_out(o[i:i + 1], ref, "gqa_xKV_rope wide, sequence %d" % i)
 
 
 def test_config1_shape_factorized_rope(dev):
