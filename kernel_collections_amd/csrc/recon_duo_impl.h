@@ -258,46 +258,6 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
   const bool sm_valid = wave < G;
   const int sm_row = sm_valid ? wave : G - 1;
   float m_ref = NEG_INF, l_run = 0.f;
-  auto softmax_tile = [&](int t) {   // scores of tile t -> P (operand type) and the rescale factor, through LDS
-    const float* sp = s_part + sm_row * FSP_ROW + 2 * n16;
-    f32x2d v[NW];
-#pragma unroll
-    for (int w = 0; w < NW; ++w) v[w] = *reinterpret_cast<const f32x2d*>(sp + w * 8 * FSP_ROW);
-    float s0 = ((v[0][0] + v[1][0]) + (v[2][0] + v[3][0])) + ((v[4][0] + v[5][0]) + (v[6][0] + v[7][0]));
-    float s1 = ((v[0][1] + v[1][1]) + (v[2][1] + v[3][1])) + ((v[4][1] + v[5][1]) + (v[6][1] + v[7][1]));
-    const int tok = start + t * FT + 2 * n16;
-    if (SCORES) {
-      if (sm_valid && lane < 16) {
-        const int64_t o = ((int64_t)b * p.hq + h0 + wave) * p.kv_len + tok;
-        s0 *= p.sm_scale;
-        s1 *= p.sm_scale;
-        if (p.scores_dtype == XKV_F32) {
-          float* dst = reinterpret_cast<float*>(p.scores) + o;
-          if (tok < end) dst[0] = s0;
-          if (tok + 1 < end) dst[1] = s1;
-        } else {
-          T* dst = reinterpret_cast<T*>(p.scores) + o;
-          if (tok < end) dst[0] = from_f32<T>(s0);
-          if (tok + 1 < end) dst[1] = from_f32<T>(s1);
-        }
-      }
-      return;
-    }
-    s0 = s0 * p.sm_scale + (tok < end ? 0.f : NEG_INF);       // (finite) - inf = -inf: masked without a branch
-    s1 = s1 * p.sm_scale + (tok + 1 < end ? 0.f : NEG_INF);
-    // the reference maximum only moves when the tile maximum exceeds it by LAZY_RESCALE (branch-free: alpha = 1 otherwise)
-    const float mx = row_reduce<true, 16>(fmaxf(s0, s1));
-    const float m_new = mx > m_ref + LAZY_RESCALE ? mx : m_ref;
-    const float alpha = __expf(m_ref - m_new);
-    m_ref = m_new;
-    const float e0 = __expf(s0 - m_ref), e1 = __expf(s1 - m_ref);
-    l_run = l_run * alpha + row_reduce<false, 16>(e0 + e1);
-    T* pd = p_lds + (t & 1) * (16 * FP_ROW) + wave * FP_ROW + 2 * n16;   // the four 16-lane groups store the same values; absent heads keep zeros
-    pd[0] = from_f32<T>(sm_valid ? e0 : 0.f);
-    pd[1] = from_f32<T>(sm_valid ? e1 : 0.f);
-    alpha_lds[(t & 1) * 16 + wave] = sm_valid ? alpha : 1.f;
-  };
-
   // ---- accumulators ---------------------------------------------------------------------------------------------------
   f32x4 acc[NMB];        // P.A: wave w owns value features DV/8 w .. + DV/8
 #pragma unroll
@@ -389,21 +349,87 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
     if (V2) duo_wait_vmcnt<S::WAIT_V>();   // this wave's rows of value tile t have landed
     __syncthreads();         // B1: partial scores of tile t, q^(t+1) visible; value tile t complete
     // ---- I2 ----
-    pv(PAR ^ 1);             // tile t-1 (its P and rescale factors were published before the last barrier)
-    softmax_tile(t);
-    tr_read(t);
+    // The softmax is a chain of dependent steps (LDS reads, adds, two cross-lane reductions, exponentials).  It is written
+    // out in four stages, each led by its share of the remaining reconstruction MFMAs, so that the chain runs under them.
+    constexpr int NI2 = NKS - KA, PER = (NI2 + 3) / 4;
+    auto mfmas = [&](auto stage_c) {
+      constexpr int S0 = KA + decltype(stage_c)::value * PER;
 #pragma unroll
-    for (int ks = KA; ks < NKS; ++ks) {
-      if (ks + PF < NKS) fr[ks + PF] = tile_frag(t + 1, ks + PF);
-      kn = Elem<T>::mfma32(breg[ks], fr[ks], kn);
+      for (int ks = S0; ks < S0 + PER; ++ks) {
+        if (ks < NKS) {
+          if (ks + PF < NKS) fr[ks + PF] = tile_frag(t + 1, ks + PF);
+          kn = Elem<T>::mfma32(breg[ks], fr[ks], kn);
+        }
+      }
+    };
+    float al = 1.f;
+    vec8 pb;
+    if (!SCORES) {     // P and the rescale factors of tile t-1 were published before the last barrier
+      al = alpha_lds[(PAR ^ 1) * 16 + n16];
+      pb = ld16<vec8>(p_lds + (PAR ^ 1) * (16 * FP_ROW) + n16 * FP_ROW + 8 * g4);
     }
-    // the softmax is a chain of dependent steps: deal the MFMAs out along it
+    f32x2d v[NW];
+    {
+      const float* sp = s_part + sm_row * FSP_ROW + 2 * n16;
 #pragma unroll
-    for (int i = 0; i < NKS - KA + (SCORES ? 0 : NMB); ++i) {
-      XKV_DUO_SGB(0x008, 1);
-      XKV_DUO_SGB(0x100, 2);
-      XKV_DUO_SGB(0x002, 7);
-      XKV_DUO_SGB(0x200, 1);
+      for (int w = 0; w < NW; ++w) v[w] = *reinterpret_cast<const f32x2d*>(sp + w * 8 * FSP_ROW);
+    }
+    const int tok = start + t * FT + 2 * n16;
+    XKV_DUO_FENCE();
+    // stage 0: sum the eight partial scores, scale, mask
+    mfmas(std::integral_constant<int, 0>());
+    float s0 = ((v[0][0] + v[1][0]) + (v[2][0] + v[3][0])) + ((v[4][0] + v[5][0]) + (v[6][0] + v[7][0]));
+    float s1 = ((v[0][1] + v[1][1]) + (v[2][1] + v[3][1])) + ((v[4][1] + v[5][1]) + (v[6][1] + v[7][1]));
+    float e0 = 0.f, e1 = 0.f, alpha = 1.f;
+    if (SCORES) {
+      if (sm_valid && lane < 16) {
+        const int64_t o = ((int64_t)b * p.hq + h0 + wave) * p.kv_len + tok;
+        s0 *= p.sm_scale;
+        s1 *= p.sm_scale;
+        if (p.scores_dtype == XKV_F32) {
+          float* dst = reinterpret_cast<float*>(p.scores) + o;
+          if (tok < end) dst[0] = s0;
+          if (tok + 1 < end) dst[1] = s1;
+        } else {
+          T* dst = reinterpret_cast<T*>(p.scores) + o;
+          if (tok < end) dst[0] = from_f32<T>(s0);
+          if (tok + 1 < end) dst[1] = from_f32<T>(s1);
+        }
+      }
+      XKV_DUO_FENCE();
+      mfmas(std::integral_constant<int, 1>());
+      mfmas(std::integral_constant<int, 2>());
+      mfmas(std::integral_constant<int, 3>());
+    } else {
+      s0 = s0 * p.sm_scale + (tok < end ? 0.f : NEG_INF);       // (finite) - inf = -inf: masked without a branch
+      s1 = s1 * p.sm_scale + (tok + 1 < end ? 0.f : NEG_INF);
+      XKV_DUO_FENCE();
+      // stage 1: the tile maximum of this head; the reference only moves when it exceeds it by LAZY_RESCALE
+      mfmas(std::integral_constant<int, 1>());
+      const float mx = row_reduce<true, 16>(fmaxf(s0, s1));
+      const float m_new = mx > m_ref + LAZY_RESCALE ? mx : m_ref;
+      XKV_DUO_FENCE();
+      // stage 2: exponentials, P and the rescale factor -> LDS (buffer t & 1; absent heads keep zeros)
+      mfmas(std::integral_constant<int, 2>());
+      alpha = __expf(m_ref - m_new);
+      m_ref = m_new;
+      e0 = __expf(s0 - m_ref);
+      e1 = __expf(s1 - m_ref);
+      T* pd = p_lds + PAR * (16 * FP_ROW) + wave * FP_ROW + 2 * n16;   // the four 16-lane groups store the same values
+      pd[0] = from_f32<T>(sm_valid ? e0 : 0.f);
+      pd[1] = from_f32<T>(sm_valid ? e1 : 0.f);
+      alpha_lds[PAR * 16 + wave] = sm_valid ? alpha : 1.f;
+      XKV_DUO_FENCE();
+      // stage 3: acc += P.A of tile t-1 from the operands in registers, then tile t's operands replace them
+      mfmas(std::integral_constant<int, 3>());
+#pragma unroll
+      for (int mb = 0; mb < NMB; ++mb) {
+        const vec8 a = __builtin_bit_cast(vec8, (s16x8d)__builtin_shufflevector(tr[2 * mb], tr[2 * mb + 1], 0, 1, 2, 3, 4, 5, 6, 7));
+        acc[mb] = Elem<T>::mfma16(a, pb, acc[mb] * al);
+      }
+      XKV_DUO_FENCE();
+      tr_read(t);
+      l_run = l_run * alpha + row_reduce<false, 16>(e0 + e1);
     }
     XKV_DUO_FENCE();
     duo_wait_vmcnt<S::WAIT_K>();   // this wave's rows of key tile t+2 have landed
