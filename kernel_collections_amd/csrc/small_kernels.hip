@@ -148,11 +148,22 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     const TB* __restrict__ vB, int64_t sVb, int64_t sVh, int64_t sVr, int d_out,
     const int32_t* __restrict__ num_kv_splits, const int32_t* __restrict__ kv_lens,
     int hq, int hkv, int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, int hpw,
-    float* __restrict__ lse_out, int64_t sLb, int64_t sLh) {
+    float* __restrict__ lse_out, int64_t sLb, int64_t sLh, int d_blk) {
   extern __shared__ float merged[];  // [G][dv], then the split weights [G][max_splits]
   __shared__ float fin[4 * 512];     // per-head-block totals of the up-projection
   // this workgroup: heads hfirst .. hfirst + G - 1 of sequence b, all of kv head kh (G = hpw divides the GQA group size)
   const int G = hpw, hfirst = blockIdx.x * hpw, kh = hfirst / (hq / hkv), b = blockIdx.y;
+  // blockIdx.z: a block of d_blk output columns of the up-projection (every block repeats the merge: when the grid is
+  // small the partial rows are read from more CUs at once, which is what bounds a single long sequence)
+  if (blockIdx.z > 0) {
+    const int cz = blockIdx.z * d_blk;
+    vB += cz;
+    out += cz;
+    d_out = d_out - cz < d_blk ? d_out - cz : d_blk;
+    lse_out = nullptr;
+  } else if (d_blk < d_out) {
+    d_out = d_blk;
+  }
   const int L = kv_lens ? kv_lens[b] : kv_len;
   const int ns = num_kv_splits[b];
   float* wts = merged + G * dv;
@@ -324,9 +335,13 @@ static int launch_merge(const float* partial, const float* lse, void* out, const
   // partial rows of a long sequence are spread over more CUs
   const int hpw = (max_splits > 16 || hq / hkv > 16) ? 1 : hq / hkv;
   size_t shm = (size_t)hpw * (dv + max_splits) * sizeof(float);
-  merge_stage2_kernel<O, TB><<<dim3(hq / hpw, batch), dim3(256), shm, st>>>(partial, lse, (O*)out, (const TB*)vB, sVb, sVh,
-                                                                           sVr, d_out, ns, kl, hq, hkv, kv_len, max_splits,
-                                                                           dv, sOb, sOh, hpw, lse_out, sLb, sLh);
+  // a small grid over many splits is bound by the latency of its partial-row loads: split the up-projection's columns
+  // over more workgroups
+  int zb = 1;
+  if (vB && (hq / hpw) * batch < 128 && max_splits >= 64 && d_out % 32 == 0) zb = d_out >= 512 ? 4 : d_out >= 256 ? 2 : 1;
+  merge_stage2_kernel<O, TB><<<dim3(hq / hpw, batch, zb), dim3(256), shm, st>>>(partial, lse, (O*)out, (const TB*)vB, sVb, sVh,
+                                                                               sVr, d_out, ns, kl, hq, hkv, kv_len, max_splits,
+                                                                               dv, sOb, sOh, hpw, lse_out, sLb, sLh, d_out / zb);
   return launch_status();
 }
 
