@@ -245,7 +245,7 @@ def bench_c4(args, dev, vfact):
     q = randn_dev((B, Hq, d), 1.0, dev, gen=gen)
     o = torch.empty_like(q)
     if vfact:
-        split = args.splits or 2048   # one workgroup serves all 32 heads of a split, so the splits are shorter than plain GQA's
+        split = args.splits or split  # the wrapper cuts long splits itself (one workgroup serves all 32 heads of a split)
     elif args.splits:
         split = args.splits
     ns_l = [-(-n // split) for n in lens]

@@ -10,7 +10,32 @@ Split ranges follow gqa.py:95-99 exactly; ``sm_scale`` multiplies the scores (gq
 """
 from __future__ import annotations
 
+import torch
+
 from kernel_collections_amd import ops
+
+
+REFINE_TOKENS = 1024   # decode_attention_fwd: longest split it runs as one workgroup (0: always the caller's splits)
+
+
+_refined = {}
+
+
+def _refine_splits(splits, lens, batch, kv_len, S, tokens, device):
+    """At least one split per `tokens` tokens for every sequence: ``max(splits, ceil(len / tokens))`` on the device (no
+    host synchronisation) and the matching bound on the split count.  The result is remembered for as long as the same
+    tensors are passed again unmodified (their version counters are part of the key), which is what a decode loop does."""
+    S2 = max(S, -(-kv_len // tokens))
+    if lens is None:
+        return torch.maximum(splits, ops.uniform_splits(batch, -(-kv_len // tokens), device)), S2
+    key = (splits.data_ptr(), splits._version, lens.data_ptr(), lens._version, tokens)
+    hit = _refined.get(key)
+    if hit is None:
+        if len(_refined) >= 16:
+            _refined.clear()
+        hit = torch.maximum(splits, ((lens + (tokens - 1)) // tokens).to(torch.int32))
+        _refined[key] = hit
+    return hit, S2
 
 
 def _prep(q, k_buffer, num_kv_splits, max_kv_splits, kv_lens):
@@ -38,6 +63,10 @@ def decode_attention_fwd(q, k_buffer, v_buffer, o, num_kv_splits, max_kv_splits,
     kv_len = k_buffer.shape[1]
     q3 = ops._q3(q)
     k_buffer, v_buffer = ops.as_rows(k_buffer), ops.as_rows(v_buffer)
+    if REFINE_TOKENS and kv_len > S * REFINE_TOKENS:
+        # shorter splits balance a ragged batch over the CUs (split-K is exact under the merge, so the caller's split
+        # count is a lower bound, not a contract on the arithmetic); computed on the device, no host synchronisation
+        splits, S = _refine_splits(splits, lens, batch, kv_len, S, REFINE_TOKENS, q.device)
     partial, lse = ops.workspaces(batch, hq, S, dv, q.device)
     ops.latent_stage1(q3, None, None,
                       (k_buffer, k_buffer.stride(0), k_buffer.stride(1), k_buffer.stride(2), d), None,
@@ -57,9 +86,17 @@ def decode_attention_fwd_v_factorized(q, k_buffer, v_A_buffer, v_B_buffer, o, nu
     kv_len = k_buffer.shape[1]
     q3 = ops._q3(q)
     k_buffer, v_A_buffer = ops.as_rows(k_buffer), ops.as_rows(v_A_buffer)
-    partial, lse = ops.workspaces(batch, hq, S, rv, q.device)
     wide = (hkv * d == 1024 and rv in (256, 384, 512)) or (hkv * d == 512 and rv == 512)
-    if wide and hq <= 32 and k_buffer.stride(2) == d:
+    wide = wide and hq <= 32 and k_buffer.stride(2) == d
+    if wide:
+        # One workgroup serves every head of a split, so there are hkv times fewer workgroups than in the per-head
+        # form: when the caller's splits are longer than 2048 tokens every sequence gets at least one split per 2048
+        # tokens (split-K is exact under the merge, so the caller's split count is a lower bound, not a contract on
+        # the arithmetic).  Computed on the device: no host synchronisation.
+        if kv_len > S * 2048:
+            splits, S = _refine_splits(splits, lens, batch, kv_len, S, 2048, q.device)
+    partial, lse = ops.workspaces(batch, hq, S, rv, q.device)
+    if wide:
         # all heads from one workgroup: the token's keys are one hkv*d-wide row against a block-diagonal query, and the
         # value basis (shared by the heads) is read once per token instead of once per kv head
         qbd = ops.blockdiag_q(q3, hkv)

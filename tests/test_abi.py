@@ -130,3 +130,23 @@ def test_settled_splits_leaves_no_dead_split():
             assert 1 <= s <= n
             live = oracle.live_splits(L, s, s)
             assert len(live) == s and live[0][1] == 0 and live[-1][2] == L, (L, n, s)
+
+
+def test_refined_splits_follow_the_lengths_and_their_updates():
+    """The plain and V-factorised decode wrappers give every sequence at least one split per N tokens; the device-side
+    result is remembered only while the caller's tensors are unmodified."""
+    from kernel_collections_amd.flash_decoding import gqa
+    lens = torch.tensor([1, 1024, 1025, 5000, 104212], dtype=torch.int32)
+    splits = torch.tensor([1, 1, 1, 2, 26], dtype=torch.int32)
+    out, S = gqa._refine_splits(splits, lens, 5, 104212, 26, 1024, lens.device)
+    assert out.dtype == torch.int32 and out.tolist() == [1, 1, 2, 5, 102] and S == 102
+    again, _ = gqa._refine_splits(splits, lens, 5, 104212, 26, 1024, lens.device)
+    assert again is out                                   # same tensors, same versions: no new device work
+    lens[3] = 9000                                        # an in-place update must not see the remembered result
+    out2, _ = gqa._refine_splits(splits, lens, 5, 104212, 26, 1024, lens.device)
+    assert out2.tolist() == [1, 1, 2, 9, 102]
+    splits[0] = 7                                         # the caller's own count is a lower bound
+    out3, S3 = gqa._refine_splits(splits, lens, 5, 104212, 200, 1024, lens.device)
+    assert out3.tolist() == [7, 1, 2, 9, 102] and S3 == 200
+    uni, Su = gqa._refine_splits(torch.full((3,), 2, dtype=torch.int32), None, 3, 5000, 2, 2048, lens.device)
+    assert uni.tolist() == [3, 3, 3] and Su == 3
