@@ -15,7 +15,8 @@ import torch
 from kernel_collections_amd import ops
 
 
-REFINE_TOKENS = 1024   # decode_attention_fwd: longest split it runs as one workgroup (0: always the caller's splits)
+REFINE_TOKENS = 1024        # decode_attention_fwd: longest split it runs as one workgroup (0: always the caller's splits)
+REFINE_TOKENS_WIDE = 2048   # the same for the all-heads form of decode_attention_fwd_v_factorized
 
 
 _refined = {}
@@ -93,8 +94,8 @@ def decode_attention_fwd_v_factorized(q, k_buffer, v_A_buffer, v_B_buffer, o, nu
         # form: when the caller's splits are longer than 2048 tokens every sequence gets at least one split per 2048
         # tokens (split-K is exact under the merge, so the caller's split count is a lower bound, not a contract on
         # the arithmetic).  Computed on the device: no host synchronisation.
-        if kv_len > S * 2048:
-            splits, S = _refine_splits(splits, lens, batch, kv_len, S, 2048, q.device)
+        if REFINE_TOKENS_WIDE and kv_len > S * REFINE_TOKENS_WIDE:
+            splits, S = _refine_splits(splits, lens, batch, kv_len, S, REFINE_TOKENS_WIDE, q.device)
     partial, lse = ops.workspaces(batch, hq, S, rv, q.device)
     if wide:
         # all heads from one workgroup: the token's keys are one hkv*d-wide row against a block-diagonal query, and the
