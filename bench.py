@@ -335,15 +335,46 @@ def bench_qabrope(args, dev):
     }
 
 
+def bench_ropedecode(args, dev):
+    """Fused xKV decode with RoPE and SEPARATE key / value bases at the default shape of the reference's variant table
+    (test_attention_profiling.py:511-517): batch 1, 32 q / 8 kv heads, head_dim 128, kv_len 131072, K rank 384, V rank 512."""
+    import kernel_collections_amd.flash_recontruction as fr
+    from kernel_collections_amd import ops
+    B, Hq, Hkv, d, L, rk, rv, theta = 1, 32, 8, 128, 131072, args.rank if args.rank != 192 else 384, 512, 5e5
+    gen = torch.Generator(device=dev).manual_seed(0)
+    q = randn_dev((B, Hq, d), 1.0, dev, torch.bfloat16, gen)
+    kA, vA = randn_dev((B, L, rk), 1.0, dev, torch.bfloat16, gen), randn_dev((B, L, rv), 1.0, dev, torch.bfloat16, gen)
+    kB = randn_dev((B, Hkv, rk, d), rk ** -0.5, dev, torch.bfloat16, gen)
+    vB = randn_dev((B, Hkv, rv, d), rv ** -0.5, dev, torch.bfloat16, gen)
+    o = torch.empty_like(q)
+    S = args.splits or ops.occupancy_splits(B, Hkv, L, tile=32, waves=1)
+    ns = ops.uniform_splits(B, S, dev)
+    total_ms = time_loop(lambda i: fr.gqa_xKV_rope(q, kA, kB, vA, vB, o, ns, S, d ** -0.5, theta), args.steps, args.warmup)
+    us = total_ms * 1e3 / args.steps
+    flops = B * L * (2 * rk * Hkv * d + 2 * Hq * d + 2 * Hq * rv)
+    tf = flops / (us * 1e-6) / 1e12
+    return {
+        "metric": "us_per_layer_decode_step", "value": round(us, 2), "unit": "us", "higher_is_better": False,
+        "ms_per_step": total_ms / args.steps,
+        "config": {"workload": "fused RoPE xKV decode, separate bases: batch 1, 32q/8kv, d128, kv_len %d, K rank %d, V rank %d, bf16"
+                               % (L, rk, rv), "kv_splits": S},
+        "roofline": {"bound": "mfma", "kernel": "recon_duo_kernel", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "note": "whole call (pack, stage 1, merge) over algorithmic FLOP", "algorithmic_flop": flops,
+                     "hbm_side_GBps": round(B * L * (rk + rv) * 2 / (us * 1e-6) / 1e9, 1)},
+        "cpu_baseline": None,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=25)
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c4v", "c5", "pdsep", "qabrope"])
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c4v", "c5", "pdsep", "qabrope", "ropedecode"])
     ap.add_argument("--ctx", type=int, default=32768)
     ap.add_argument("--splits", type=int, default=0)
-    ap.add_argument("--rank", type=int, default=192, help="rank of the qabrope workload")
+    ap.add_argument("--rank", type=int, default=192, help="rank of the qabrope workload (ropedecode: K rank, default 384)")
     ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16"], help="operand type of the qabrope workload")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-comparator", action="store_true")
@@ -374,6 +405,8 @@ def main():
         res = bench_pdsep(args, dev)
     elif args.config == "qabrope":
         res = bench_qabrope(args, dev)
+    elif args.config == "ropedecode":
+        res = bench_ropedecode(args, dev)
     else:
         res = bench_c4(args, dev, args.config == "c4v")
     line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"), "n_gpus": 1,
