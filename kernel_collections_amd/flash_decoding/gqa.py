@@ -10,6 +10,8 @@ Split ranges follow gqa.py:95-99 exactly; ``sm_scale`` multiplies the scores (gq
 """
 from __future__ import annotations
 
+import weakref
+
 import torch
 
 from kernel_collections_amd import ops
@@ -19,24 +21,26 @@ REFINE_TOKENS = 1024        # decode_attention_fwd: longest split it runs as one
 REFINE_TOKENS_WIDE = 2048   # the same for the all-heads form of decode_attention_fwd_v_factorized
 
 
-_refined = {}
+_refined = {}   # (id(splits), id(lens), tokens) -> (weakref(splits), weakref(lens), versions, result)
 
 
 def _refine_splits(splits, lens, batch, kv_len, S, tokens, device):
     """At least one split per `tokens` tokens for every sequence: ``max(splits, ceil(len / tokens))`` on the device (no
-    host synchronisation) and the matching bound on the split count.  The result is remembered for as long as the same
-    tensors are passed again unmodified (their version counters are part of the key), which is what a decode loop does."""
+    host synchronisation) and the matching bound on the split count.  The result is remembered while the SAME tensor
+    objects are passed again unmodified (identity through weak references, so a freed tensor whose address is reused
+    never matches, plus the tensors' version counters), which is what a decode loop does."""
     S2 = max(S, -(-kv_len // tokens))
     if lens is None:
         return torch.maximum(splits, ops.uniform_splits(batch, -(-kv_len // tokens), device)), S2
-    key = (splits.data_ptr(), splits._version, lens.data_ptr(), lens._version, tokens)
+    key = (id(splits), id(lens), tokens)
     hit = _refined.get(key)
-    if hit is None:
-        if len(_refined) >= 16:
-            _refined.clear()
-        hit = torch.maximum(splits, ((lens + (tokens - 1)) // tokens).to(torch.int32))
-        _refined[key] = hit
-    return hit, S2
+    if hit is not None and hit[0]() is splits and hit[1]() is lens and hit[2] == (splits._version, lens._version):
+        return hit[3], S2
+    if len(_refined) >= 16:
+        _refined.clear()
+    out = torch.maximum(splits, ((lens + (tokens - 1)) // tokens).to(torch.int32))
+    _refined[key] = (weakref.ref(splits), weakref.ref(lens), (splits._version, lens._version), out)
+    return out, S2
 
 
 def _prep(q, k_buffer, num_kv_splits, max_kv_splits, kv_lens):

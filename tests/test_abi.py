@@ -148,5 +148,8 @@ def test_refined_splits_follow_the_lengths_and_their_updates():
     splits[0] = 7                                         # the caller's own count is a lower bound
     out3, S3 = gqa._refine_splits(splits, lens, 5, 104212, 200, 1024, lens.device)
     assert out3.tolist() == [7, 1, 2, 9, 102] and S3 == 200
+    other = torch.tensor([4000, 10, 10, 10, 10], dtype=torch.int32)    # another tensor object never sees a remembered result
+    out4, _ = gqa._refine_splits(splits, other, 5, 104212, 26, 1024, lens.device)
+    assert out4.tolist() == [7, 1, 1, 2, 26]
     uni, Su = gqa._refine_splits(torch.full((3,), 2, dtype=torch.int32), None, 3, 5000, 2, 2048, lens.device)
     assert uni.tolist() == [3, 3, 3] and Su == 3
