@@ -43,7 +43,10 @@ constexpr int FT = 32;              // tokens per tile
 constexpr int NW = 8;               // wavefronts per workgroup
 constexpr int FSP_ROW = FT + 4;     // partial-score row stride (floats)
 constexpr int FP_ROW = FT + 8;      // P row stride (elements)
-constexpr float LAZY_RESCALE = 16.f; // the softmax reference only moves when a tile maximum exceeds it by this much
+// The softmax reference only moves when a tile maximum exceeds it by this much.  P = exp(s - reference) is stored in the
+// operand type, so the bound must keep exp(bound) finite there: e^16 = 8.9e6 fits bf16's exponent range, but fp16 ends
+// at 65504 = e^11.09, hence 8 (e^8 = 2981) for fp16.
+template <typename T> constexpr float lazy_rescale() { return std::is_same<T, _Float16>::value ? 8.f : 16.f; }
 #define XKV_DUO_FENCE() __builtin_amdgcn_sched_barrier(0)
 #define XKV_DUO_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)   // 0x8 MFMA, 0x2 VALU, 0x100 LDS read, 0x200 LDS write
 
@@ -197,8 +200,8 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
   unsigned char* kring = smem;                                             // NSK * KTILE
   unsigned char* vring = V2 ? smem + NSK * KTILE : smem;                   // NSV * VTILE (one stream: the key ring)
   float* s_part = reinterpret_cast<float*>(smem + NSK * KTILE + NSV * VTILE);   // [8 waves][8 heads][FSP_ROW]
-  T* qhat = reinterpret_cast<T*>(s_part + NW * 8 * FSP_ROW);               // [2][8 heads][128]
-  T* p_lds = qhat + 2 * 8 * 128;                                           // [2][16 head slots][FP_ROW]
+  sc_t* qhat = reinterpret_cast<sc_t*>(s_part + NW * 8 * FSP_ROW);         // [2][8 heads][128]
+  T* p_lds = reinterpret_cast<T*>(qhat + 2 * 8 * 128);                                          // [2][16 head slots][FP_ROW]
   float* alpha_lds = reinterpret_cast<float*>(p_lds + 2 * 16 * FP_ROW);    // [2][16]
   float* ml_lds = alpha_lds + 32;                                          // [8][2]
   const unsigned smem_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)smem;
@@ -247,9 +250,9 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
   auto write_qhat = [&](int t) {   // q^ for tile t = R(-base(t)) q, into buffer t & 1
     if ((t & 31) == 0)             // the base advances by angle addition; every 32 tiles it is range-reduced afresh
       sincosf((float)(p.pos_offset + start + (int64_t)t * FT) * qinv, &qsb, &qcb);
-    T* dst = qhat + (t & 1) * (8 * 128) + wave * 128 + qpos;
-    dst[0] = from_f32<T>(q0 * qcb + q1 * qsb);
-    dst[4] = from_f32<T>(q1 * qcb - q0 * qsb);
+    sc_t* dst = qhat + (t & 1) * (8 * 128) + wave * 128 + qpos;
+    dst[0] = from_f32<sc_t>(q0 * qcb + q1 * qsb);
+    dst[4] = from_f32<sc_t>(q1 * qcb - q0 * qsb);
     const float c = qcb * qc32 - qsb * qs32, s = qsb * qc32 + qcb * qs32;
     qcb = c; qsb = s;
   };
@@ -270,7 +273,7 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
   auto tile_frag = [&](int t, int ks) -> vec8 {
     return ld16<vec8>(kring + (t % NSK) * KTILE + n32 * KROW + ((RK / 2) * kq + 8 * g2) * 2 + ks * 32);
   };
-  const T* qrow = qhat + (n32 < G ? n32 : G - 1) * 128 + (dq * 4 + g2) * 8;
+  const sc_t* qrow = qhat + (n32 < G ? n32 : G - 1) * 128 + (dq * 4 + g2) * 8;
   auto tr_read = [&](int t) {   // this wave's DV/8 value features of tile t, token-major
     if (SCORES) return;
     constexpr int VR = V2 ? VROW : KROW;
@@ -312,9 +315,9 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
     vec8 fr[NKS];
 #pragma unroll
     for (int i = 0; i < PF; ++i) fr[i] = tile_frag(t + 1, i);
-    const T* qr = qrow + PAR * (8 * 128);
-    const vec8 qop0 = ld16<vec8>(qr), qop1 = ld16<vec8>(qr + 16);
-    vec8 kop[2];
+    const sc_t* qr = qrow + PAR * (8 * 128);
+    const sc_vec8 qop0 = ld16<sc_vec8>(qr), qop1 = ld16<sc_vec8>(qr + 16);
+    sc_vec8 kop[2];
     f32x16 sacc;
 #pragma unroll
     for (int ks = 0; ks < KA; ++ks) {
@@ -322,14 +325,14 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
 #pragma unroll
         for (int r = 2 * ks; r < 2 * ks + 2; ++r) {
           const int o = r >> 2, e = r & 3;
-          kop[o][e] = from_f32<T>(kc[r] * ci[r] - kc[r + 8] * si[r]);
-          kop[o][4 + e] = from_f32<T>(kc[r + 8] * ci[r] + kc[r] * si[r]);
+          kop[o][e] = from_f32<sc_t>(kc[r] * ci[r] - kc[r + 8] * si[r]);
+          kop[o][4 + e] = from_f32<sc_t>(kc[r + 8] * ci[r] + kc[r] * si[r]);
         }
       }
       if (ks + PF < NKS) fr[ks + PF] = tile_frag(t + 1, ks + PF);
       kn = Elem<T>::mfma32(breg[ks], fr[ks], ks == 0 ? z16 : kn);
-      if (ks == 1) sacc = Elem<T>::mfma32(kop[0], qop0, z16);
-      if (ks == 3) sacc = Elem<T>::mfma32(kop[1], qop1, sacc);
+      if (ks == 1) sacc = Elem<sc_t>::mfma32(kop[0], qop0, z16);
+      if (ks == 3) sacc = Elem<sc_t>::mfma32(kop[1], qop1, sacc);
       if (ks == 2) {             // scalar address work and the load issue run under the MFMAs already in the pipe
         XKV_DUO_FENCE();
         ks_.issue(end, last, wave, lane);          // key tile t + KAHEAD, into the slot freed at the last barrier
@@ -404,10 +407,10 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
       s0 = s0 * p.sm_scale + (tok < end ? 0.f : NEG_INF);       // (finite) - inf = -inf: masked without a branch
       s1 = s1 * p.sm_scale + (tok + 1 < end ? 0.f : NEG_INF);
       XKV_DUO_FENCE();
-      // stage 1: the tile maximum of this head; the reference only moves when it exceeds it by LAZY_RESCALE
+      // stage 1: the tile maximum of this head; the reference only moves when it exceeds it by lazy_rescale<T>()
       mfmas(std::integral_constant<int, 1>());
       const float mx = row_reduce<true, 16>(fmaxf(s0, s1));
-      const float m_new = mx > m_ref + LAZY_RESCALE ? mx : m_ref;
+      const float m_new = mx > m_ref + lazy_rescale<T>() ? mx : m_ref;
       XKV_DUO_FENCE();
       // stage 2: exponentials, P and the rescale factor -> LDS (buffer t & 1; absent heads keep zeros)
       mfmas(std::integral_constant<int, 2>());

@@ -47,7 +47,10 @@ constexpr int FTILE = FT * FROW;    // 33280
 constexpr int FRING = 4;
 constexpr int FSP_ROW = FT + 4;     // partial-score row stride (floats)
 constexpr int FP_ROW = FT + 8;      // P row stride (elements)
-constexpr float LAZY_RESCALE = 16.f; // the softmax reference only moves when a tile maximum exceeds it by this much
+// The softmax reference only moves when a tile maximum exceeds it by this much.  P = exp(s - reference) is stored in the
+// operand type, so the bound must keep exp(bound) finite there: e^16 = 8.9e6 fits bf16's exponent range, but fp16 ends
+// at 65504 = e^11.09, hence 8 (e^8 = 2981) for fp16.
+template <typename T> constexpr float lazy_rescale() { return std::is_same<T, _Float16>::value ? 8.f : 16.f; }
 
 // The LDS destination of a direct-to-LDS load is M0 + lane * 16.  A SALU write of M0 needs one wait state
 // before an instruction that reads M0 (the compiler schedules around this for its own code; here it is explicit).
@@ -124,8 +127,8 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   // ---- LDS carve-up ---------------------------------------------------------------------------------------------
   unsigned char* ring = smem;                                              // FRING * FTILE
   float* s_part = reinterpret_cast<float*>(smem + FRING * FTILE);          // [4 waves][8 heads][FSP_ROW]
-  T* qhat = reinterpret_cast<T*>(s_part + 4 * 8 * FSP_ROW);                // [2][8 heads][128]
-  T* p_lds = qhat + 2 * 8 * 128;                                           // [16 head slots][FP_ROW]
+  sc_t* qhat = reinterpret_cast<sc_t*>(s_part + 4 * 8 * FSP_ROW);          // [2][8 heads][128]
+  T* p_lds = reinterpret_cast<T*>(qhat + 2 * 8 * 128);                                          // [16 head slots][FP_ROW]
   float* alpha_lds = reinterpret_cast<float*>(p_lds + 16 * FP_ROW);        // [16]
   float* ml_lds = alpha_lds + 16;                                          // [8][2]
   const unsigned ring_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)ring;
@@ -212,11 +215,11 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     const bool sd = t == seed_t;
     qcb = sd ? seed_c : qcb;
     qsb = sd ? seed_s : qsb;
-    T* dst = qhat + (t & 1) * (8 * 128) + wave * 128 + qpos;
+    sc_t* dst = qhat + (t & 1) * (8 * 128) + wave * 128 + qpos;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      dst[i * 512] = from_f32<T>(q0[i] * qcb + q1[i] * qsb);
-      dst[i * 512 + 4] = from_f32<T>(q1[i] * qcb - q0[i] * qsb);
+      dst[i * 512] = from_f32<sc_t>(q0[i] * qcb + q1[i] * qsb);
+      dst[i * 512 + 4] = from_f32<sc_t>(q1[i] * qcb - q0[i] * qsb);
     }
     const float c = qcb * qc32 - qsb * qs32, s = qsb * qc32 + qcb * qs32;
     qcb = c; qsb = s;
@@ -258,12 +261,12 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     }
     s0 = tok < end ? s0 * p.sm_scale : NEG_INF;
     s1 = tok + 1 < end ? s1 * p.sm_scale : NEG_INF;
-    // the reference maximum only moves when the tile maximum exceeds it by LAZY_RESCALE; the reduction that finds the
+    // the reference maximum only moves when the tile maximum exceeds it by lazy_rescale<T>(); the reduction that finds the
     // maximum runs only then, so the usual path from scores to P has no cross-lane step
     float alpha = 1.f;
-    if (__builtin_amdgcn_ballot_w64(fmaxf(s0, s1) > m_ref + LAZY_RESCALE)) {   // rare: some head's maximum moves
+    if (__builtin_amdgcn_ballot_w64(fmaxf(s0, s1) > m_ref + lazy_rescale<T>())) {   // rare: some head's maximum moves
       const float mx = row_reduce<true, 16>(fmaxf(s0, s1));
-      const float m_new = mx > m_ref + LAZY_RESCALE ? mx : m_ref;
+      const float m_new = mx > m_ref + lazy_rescale<T>() ? mx : m_ref;
       alpha = __expf(m_ref - m_new);
       m_ref = m_new;
     }
@@ -281,7 +284,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   for (int mb = 0; mb < 8; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
   f32x16 ka[2][2];       // two sets of partial key accumulators [set][low | partner feature block]
   vec8 at[16];           // this wave's 16 rank chunks of the tile being reconstructed (read one part ahead of their use)
-  vec8 qop[4];           // q^ operands of the tile being rotated
+  sc_vec8 qop[4];        // q^ operands of the tile being rotated
 
   auto tile_frag = [&](int t, int ks) -> vec8 {
     return ld16<vec8>(ring + (t & (FRING - 1)) * FTILE + n32 * FROW + (256 * kq + 8 * g2) * 2 + ks * 32);
@@ -330,18 +333,18 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
           }
         }
         if (DO_PREV) {
-          vec8 kop;
+          sc_vec8 kop;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int r = 4 * o + e;
-            kop[e] = from_f32<T>(j0[r] * ci[r] - j1[r] * si[r]);
-            kop[4 + e] = from_f32<T>(j1[r] * ci[r] + j0[r] * si[r]);
+            kop[e] = from_f32<sc_t>(j0[r] * ci[r] - j1[r] * si[r]);
+            kop[4 + e] = from_f32<sc_t>(j1[r] * ci[r] + j0[r] * si[r]);
           }
           if (o == 0) {
             const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            sacc = Elem<T>::mfma32(kop, qop[o], z);
+            sacc = Elem<sc_t>::mfma32(kop, qop[o], z);
           } else {
-            sacc = Elem<T>::mfma32(kop, qop[o], sacc);
+            sacc = Elem<sc_t>::mfma32(kop, qop[o], sacc);
           }
         }
         if (DO_R && DO_PREV) {   // three reconstruction MFMAs dealt out among the rotation's VALU work, then the q-dot
@@ -407,8 +410,9 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
                             // the transposed reads of tile i-1 have returned, so its ring slot is free
     // ---- part 3 ----------------------------------------------------------------------------------------------------------
     vec8 pb;
-    vec8 at_next[6], qop_next[4];
-    const T* qrow = qhat + (i & 1) * (8 * 128) + (n32 < G ? n32 : G - 1) * 128 + (dq * 2 + g2) * 8;
+    vec8 at_next[6];
+    sc_vec8 qop_next[4];
+    const sc_t* qrow = qhat + (i & 1) * (8 * 128) + (n32 < G ? n32 : G - 1) * 128 + (dq * 2 + g2) * 8;
     auto pv_step = [&](int mb) {
       if (SCORES) return;
       vec8 a = __builtin_bit_cast(vec8, (s16x8f)__builtin_shufflevector(tr[2 * mb], tr[2 * mb + 1], 0, 1, 2, 3, 4, 5, 6, 7));
@@ -436,7 +440,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       if (DO_R) {
         at_next[u] = tile_frag(i + 1, u);
         if (u == 4) at_next[5] = tile_frag(i + 1, 5);
-        qop_next[u - 1] = ld16<vec8>(qrow + (u - 1) * 32);
+        qop_next[u - 1] = ld16<sc_vec8>(qrow + (u - 1) * 32);
         recon_step(11 + u);
         if (u == 1) issue_rows(i + 3, IC<0>(), IC<4>(), full_c);   // into the ring slot of tile i-1, whose readers are done
         if (u == 3) issue_rows(i + 3, IC<4>(), IC<8>(), full_c);

@@ -95,13 +95,13 @@ __global__ __launch_bounds__(256) void recon_stage1_kernel(const ReconParams p) 
       breg[ks][mb] = v;
     }
   // q operand of the q-dot: lane (n16 = head, g4) holds q[head][4 low features | 4 partner features]
-  vec8 qop = {0, 0, 0, 0, 0, 0, 0, 0};
+  sc_vec8 qop = {0, 0, 0, 0, 0, 0, 0, 0};
   if (n16 < G) {
     const T* qh = reinterpret_cast<const T*>(p.q) + ((int64_t)b * p.hq + h0 + n16) * 128;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      qop[e] = qh[16 * wave + 4 * g4 + e];
-      qop[4 + e] = qh[64 + 16 * wave + 4 * g4 + e];
+      qop[e] = from_f32<sc_t>(to_f32(qh[16 * wave + 4 * g4 + e]));
+      qop[4 + e] = from_f32<sc_t>(to_f32(qh[64 + 16 * wave + 4 * g4 + e]));
     }
   }
   // RoPE constants for this lane's 4 pair indices j = 16*wave + 4*g4 + r
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(256) void recon_stage1_kernel(const ReconParams p) 
           k1 = Elem<T>::mfma16(breg[ks][1], at, k1);
         }
       // lane (n16 = token, g4): k0[r] = K[token][16w+4g+r], k1[r] = K[token][64+16w+4g+r]
-      vec8 kop;
+      sc_vec8 kop;
       if (p.rope) {
         float c[4], s[4];
         if (computed_rope) {
@@ -226,15 +226,15 @@ __global__ __launch_bounds__(256) void recon_stage1_kernel(const ReconParams p) 
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          kop[r] = from_f32<T>(k0[r] * c[r] - k1[r] * s[r]);
-          kop[4 + r] = from_f32<T>(k1[r] * c[r] + k0[r] * s[r]);
+          kop[r] = from_f32<sc_t>(k0[r] * c[r] - k1[r] * s[r]);
+          kop[4 + r] = from_f32<sc_t>(k1[r] * c[r] + k0[r] * s[r]);
         }
       } else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) { kop[r] = from_f32<T>(k0[r]); kop[4 + r] = from_f32<T>(k1[r]); }
+        for (int r = 0; r < 4; ++r) { kop[r] = from_f32<sc_t>(k0[r]); kop[4 + r] = from_f32<sc_t>(k1[r]); }
       }
       f32x4 sp = {0.f, 0.f, 0.f, 0.f};
-      sp = Elem<T>::mfma16(kop, qop, sp);  // lane (n16 = head, g4): tokens tb*16 + 4*g4 + r
+      sp = Elem<sc_t>::mfma16(kop, qop, sp);  // lane (n16 = head, g4): tokens tb*16 + 4*g4 + r
       *reinterpret_cast<f32x4*>(s_part + (wave * 16 + n16) * LDS_S + tb * 16 + 4 * g4) = sp;
     }
     __syncthreads();

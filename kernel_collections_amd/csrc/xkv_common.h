@@ -43,6 +43,14 @@ template <> struct Elem<_Float16> {
 template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
 template <typename T> __device__ __forceinline__ T from_f32(float x) { return (T)x; }
 
+// The reconstruction kernels hand the rotated key tile and the query to the q-dot MFMA as fp16 WHATEVER the operand type.
+// The reference's kernels do the same (`.to(tl.float16)` before the dot, flash_recontruction/qAB/v1.py:73-74), and it
+// matters for parity: a key rounded to bf16 (8 mantissa bits) puts ~1e-3 * |s| of noise on every score, which at
+// sm_scale = 1 on unit-variance inputs (logit sigma 7 - 11, the reference scripts' regime) moves attention outputs by
+// 3e-2 .. 9e-2; fp16's 11 bits keep that below 1e-2.  Like the reference this assumes |K'| and |q| stay below 65504.
+typedef _Float16 sc_t;
+typedef f16x8 sc_vec8;
+
 __device__ __forceinline__ u16 bits_of(__bf16 x) { return __builtin_bit_cast(u16, x); }
 __device__ __forceinline__ u16 bits_of(_Float16 x) { return __builtin_bit_cast(u16, x); }
 

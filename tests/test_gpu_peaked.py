@@ -1,0 +1,213 @@
+"""GPU parity in the peaked-softmax regime, for every split-K stage-1 kernel and both operand types.
+
+The reference's own scripts run ``sm_scale = 1.0`` on unit-variance fp16 inputs: logit sigma ~ 11 for plain keys
+(test_triton_gqa.py:31-44) and ~ 7 for factorised ones drawn as ``randn / 3`` (test_gqa_xKV.py:29-36).  The scenarios:
+
+  sigma7 / sigma11  Gaussian logits of that spread at ``sm_scale = 1.0``;
+  late_max          logits of sigma ~ 2, plus, for every head, ONE token - the last token of a split, i.e. in the split's
+                    last tile - whose score is raised by 12 .. 30 (cycling over the heads), so that the running maximum
+                    moves late and by every amount around the kernels' rescale thresholds (8 for fp16, 16 for bf16) and
+                    around ln(65504) = 11.09, where exp() leaves fp16's range;
+  one_hot           the same with a raise of 45: the softmax is one-hot to fp32 precision and the output is that token's
+                    value row.
+
+The planted token's key direction is added to the query (both sides see the same rounded 16-bit query), so the values,
+and with them the outputs, stay O(1) and the absolute bar of 2e-2 means what it says.  Each path names the kernel it
+reaches; the oracle runs in fp32 on the same 16-bit-rounded inputs.
+"""
+import math
+
+import pytest
+import torch
+
+import oracle
+from util import OUT_ATOL, check_out, f32, gen, max_abs
+
+pytestmark = pytest.mark.gpu
+
+import kernel_collections_amd.flash_recontruction as fr  # noqa: E402
+from kernel_collections_amd.flash_decoding import gqa, mla2  # noqa: E402
+
+BF, FP = torch.bfloat16, torch.float16
+D = 128
+RAISES = (12.0, 15.0, 17.0, 19.0, 22.0, 30.0)
+
+
+def _splits(vals, dev):
+    return torch.tensor(vals, dtype=torch.int32, device=dev)
+
+
+def _make_q(scn, keys, hq, dtype, L, S, seed):
+    """keys ``[b, L, hkv, Dk]`` fp32: the effective (rotated, reconstructed) key of every token.  Returns q ``[b, hq, Dk]``
+    in the operand type with the scenario's logit statistics at sm_scale = 1."""
+    b, _, hkv, dk = keys.shape
+    g = hq // hkv
+    sk = keys.std().item()
+    gq = torch.Generator().manual_seed(seed)
+    base = {"sigma7": 7.0, "sigma11": 11.3}.get(scn, 2.0)
+    q = torch.randn(b, hq, dk, generator=gq) * (base / (math.sqrt(dk) * sk))
+    if scn in ("late_max", "one_hot"):
+        live = oracle.live_splits(L, S, S)
+        for ib in range(b):
+            for h in range(hq):
+                _, _, end = live[(h + ib) % len(live)]
+                k = keys[ib, end - 1, h // g]
+                raise_by = 45.0 if scn == "one_hot" else RAISES[h % len(RAISES)]
+                q[ib, h] += k * (raise_by / k.norm().item() ** 2)
+    return q.to(dtype)
+
+
+class Path:
+    """One entry point at one shape.  `inputs(dtype)` draws the 16-bit key-side operands, `keys(inp)` their effective fp32
+    keys, `run(dev, q, inp)` the HIP result and `ref(q, inp)` the oracle's."""
+    b, hq, hkv, L, S = 2, 32, 8, 1500, 4
+
+
+class ReconRope(Path):
+    theta = 5e5
+
+    def __init__(self, rk, rv, shared, table=False, hq=32, hkv=8, off=0):
+        self.rk, self.rv, self.shared, self.table, self.hq, self.hkv, self.off = rk, rv, shared, table, hq, hkv, off
+
+    def inputs(self, dtype):
+        kA = gen((self.b, self.L, self.rk), dtype=dtype, seed=2)
+        kB = gen((self.b, self.hkv, self.rk, D), std=self.rk ** -0.5, dtype=dtype, seed=3)
+        vA = kA if self.shared else gen((self.b, self.L, self.rv), dtype=dtype, seed=4)
+        vB = gen((self.b, self.hkv, vA.shape[-1], D), std=vA.shape[-1] ** -0.5, dtype=dtype, seed=5)
+        if self.table:
+            t = oracle.sin_cos_table(self.L, D, self.theta, self.off).to(dtype)
+            cos, sin = torch.cat((t[:, 64:], t[:, 64:]), -1).float(), torch.cat((t[:, :64], t[:, :64]), -1).float()
+        else:
+            t = None
+            cos, sin = oracle.rope_cos_sin(torch.arange(self.off, self.off + self.L), D, self.theta)
+        return dict(kA=kA, kB=kB, vA=vA, vB=vB, cos=cos, sin=sin, table=t)
+
+    def keys(self, i):
+        return oracle.reconstruct_rope(i["kA"].float(), i["kB"].float(), i["cos"], i["sin"]).transpose(1, 2)
+
+    def run(self, dev, q, i):
+        kA = i["kA"].to(dev)
+        vA = kA if self.shared else i["vA"].to(dev)
+        o = torch.zeros(self.b, self.hq, D, dtype=q.dtype, device=dev)
+        kw = dict(sin_cos=i["table"].to(dev)) if self.table else dict(pos_offset=self.off)
+        fr.gqa_xKV_rope(q.to(dev), kA, i["kB"].to(dev), vA, i["vB"].to(dev), o, _splits([self.S] * self.b, dev), self.S,
+                        1.0, self.theta, **kw)
+        return o
+
+    def ref(self, q, i):
+        return oracle.gqa_factorized_rope(*f32(q.unsqueeze(2), i["kA"], i["kB"], i["vA"], i["vB"]), i["cos"], i["sin"],
+                                          sm_scale=1.0)[:, :, 0]
+
+    def angle_noise(self, q, i, ref):
+        """How far the oracle's output moves when its fp32 angles ``fl(pos * inv_freq)`` (rope_ref.py:4-9) are replaced by
+        the same products in double.  Near position 128K an fp32 angle is only good to 4e-3 rad, the kernels reach the
+        same positions by angle addition from a differently rounded base, and in the peaked regime that alone moves
+        outputs by more than the parity bar; the bar is widened by what the oracle itself is uncertain by."""
+        if self.table or self.off == 0:
+            return 0.0
+        ang = torch.outer(torch.arange(self.off, self.off + self.L).double(), oracle.rope_inv_freq(D, self.theta).double())
+        ang = torch.cat((ang, ang), -1)
+        exact = self.ref(q, dict(i, cos=ang.cos().float(), sin=ang.sin().float()))
+        return (exact - ref).abs().max().item()
+
+
+class FusedNope(Path):
+    def __init__(self, rk, rv):
+        self.rk, self.rv = rk, rv
+
+    def inputs(self, dtype):
+        return dict(kA=gen((self.b, self.L, self.rk), dtype=dtype, seed=2),
+                    kB=gen((self.b, self.hkv, self.rk, D), std=self.rk ** -0.5, dtype=dtype, seed=3),
+                    vA=gen((self.b, self.L, self.rv), dtype=dtype, seed=4),
+                    vB=gen((self.b, self.hkv, self.rv, D), std=self.rv ** -0.5, dtype=dtype, seed=5))
+
+    def keys(self, i):
+        return oracle.reconstruct(i["kA"].float(), i["kB"].float()).transpose(1, 2)
+
+    def run(self, dev, q, i):
+        return fr.gqa_xKV_no_pe_v2(q.to(dev), i["kA"].to(dev), i["kB"].to(dev), i["vA"].to(dev), i["vB"].to(dev),
+                                   _splits([self.S] * self.b, dev), self.S, 1.0)
+
+    def ref(self, q, i):
+        return oracle.gqa_xkv(*f32(q, i["kA"], i["kB"], i["vA"], i["vB"]), sm_scale=1.0)
+
+
+class Plain(Path):
+    def __init__(self, v_factorised):
+        self.vf = v_factorised
+
+    def inputs(self, dtype):
+        return dict(K=gen((self.b, self.L, self.hkv, D), dtype=dtype, seed=2), V=gen((self.b, self.L, self.hkv, D), dtype=dtype, seed=3),
+                    vA=gen((self.b, self.L, 512), dtype=dtype, seed=4), vB=gen((self.b, self.hkv, 512, D), std=512 ** -0.5, dtype=dtype, seed=5))
+
+    def keys(self, i):
+        return i["K"].float()
+
+    def run(self, dev, q, i):
+        o = torch.zeros(self.b, self.hq, D, dtype=q.dtype, device=dev)
+        ns = _splits([self.S] * self.b, dev)
+        if self.vf:
+            return gqa.decode_attention_fwd_v_factorized(q.to(dev), i["K"].to(dev), i["vA"].to(dev), i["vB"].to(dev), o, ns, self.S, 1.0)
+        return gqa.decode_attention_fwd(q.to(dev), i["K"].to(dev), i["V"].to(dev), o, ns, self.S, 1.0)
+
+    def ref(self, q, i):
+        if self.vf:
+            return oracle.gqa_v_only(*f32(q.unsqueeze(2), i["K"].transpose(1, 2), i["vA"], i["vB"]), sm_scale=1.0)[:, :, 0]
+        return oracle.gqa_plain(*f32(q, i["K"], i["V"]), 1.0)
+
+
+class Mla(Path):
+    hq, hkv = 16, 1
+
+    def inputs(self, dtype):
+        return dict(ckv=gen((self.b, self.L, 1, 512), dtype=dtype, seed=2), kpe=gen((self.b, self.L, 1, 64), dtype=dtype, seed=3))
+
+    def keys(self, i):
+        return torch.cat((i["ckv"], i["kpe"]), -1).float()
+
+    def _split(self):
+        # the wrapper picks its own split count; the planted tokens only need to be last in SOME tile
+        return None
+
+    def run(self, dev, q, i):
+        return mla2.mla_decode_attention_fwd(q[..., :512].contiguous().to(dev), q[..., 512:].contiguous().to(dev),
+                                             i["ckv"].to(dev), i["kpe"].to(dev), 1.0)
+
+    def ref(self, q, i):
+        return oracle.mla_ref(*f32(q[..., :512], q[..., 512:], i["ckv"], i["kpe"]), 1.0)
+
+
+PATHS = {
+    "recon_fast(r512 shared)": ReconRope(512, 512, True),
+    "recon_fast(r512 shared, positions near 128K)": ReconRope(512, 512, True, off=131072 - 1500),
+    "recon_duo(r384/512)": ReconRope(384, 512, False),
+    "recon_duo(r512/512)": ReconRope(512, 512, False),
+    "recon_duo(r256 shared, G 8)": ReconRope(256, 256, True, hq=16, hkv=2),
+    "recon_stage1(r192 shared)": ReconRope(192, 192, True),
+    "recon_stage1(r512 table)": ReconRope(512, 512, True, table=True),
+    "latent_ring(absorbed r512/512)": FusedNope(512, 512),
+    "latent_ring(absorbed r256/384)": FusedNope(256, 384),
+    "latent_stage1(absorbed r192/64)": FusedNope(192, 64),
+    "latent_ring(mla 512+64)": Mla(),
+    "latent_ring(block-diagonal q, v_A 512)": Plain(True),
+    "latent_stage1(plain gqa)": Plain(False),
+}
+
+
+@pytest.mark.parametrize("dtype", [BF, FP], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("scn", ["sigma7", "sigma11", "late_max", "one_hot"])
+@pytest.mark.parametrize("name", list(PATHS))
+def test_peaked_softmax(dev, name, scn, dtype):
+    p = PATHS[name]
+    inp = p.inputs(dtype)
+    q = _make_q(scn, p.keys(inp), p.hq, dtype, p.L, p.S, seed=1)
+    ref = p.ref(q, inp)
+    assert torch.isfinite(ref).all()
+    out = p.run(dev, q, inp)
+    assert torch.isfinite(out.float()).all(), f"{name} / {scn}: non-finite output"
+    noise = p.angle_noise(q, inp, ref) if hasattr(p, "angle_noise") else 0.0
+    if noise == 0.0:
+        check_out(out, ref, f"{name} / {scn}")
+    else:
+        err = max_abs(out, ref)
+        assert err <= OUT_ATOL + 1.5 * noise, f"{name} / {scn}: max abs err {err:.3e} (oracle's own angle noise {noise:.3e})"
