@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define XKV_ABI_VERSION 2
+#define XKV_ABI_VERSION 3
 
 enum { XKV_F16 = 0, XKV_BF16 = 1, XKV_F32 = 2 };
 
@@ -49,6 +49,21 @@ const char* xkv_error_string(int code);
  * (angles follow the eager closed form of rope/rope_ref.py:3-9: fp32 pos * fp32 inv_freq). */
 int xkv_rope_table(void* sin_out, void* cos_out, const float* inv_freq, int64_t seqlen, int64_t start,
                    int half_dim, int out_dtype, void* stream);
+
+/* Rotate-half RoPE applied on the device, out of place or in place (out == x):
+ *   pos            = (positions ? positions[b] : pos0) + r            (positions: device int64 [batch], may be NULL)
+ *   out[b,r,h,j]        = x[b,r,h,j] * cos(a) - x[b,r,h,j+dim/2] * sin(a),   a = float(pos) * inv_freq[j]  (fp32)
+ *   out[b,r,h,j+dim/2]  = x[b,r,h,j+dim/2] * cos(a) + x[b,r,h,j] * sin(a)
+ * for x, out [batch, rows, heads, dim] with element strides (b, r, h) and a unit feature stride; dtype XKV_F32 / F16 /
+ * BF16 (arithmetic in fp32).  A decode step's query is rows == 1 at positions[b] = that sequence's length; a tail of
+ * freshly decoded keys is rows == its length at positions[b] = its first position.
+ * Replaces the eager x * cos + rotate_half(x) * sin of flash_recontruction/rope/rope_ref.py:17-20 on tables from
+ * rope_ref.py:3-9 (what the reference's callers run on the host side of every kernel that takes `q_pe`). */
+int xkv_rope_apply(const void* x, void* out, const float* inv_freq, const int64_t* positions, int64_t pos0,
+                   int batch, int rows, int heads, int dim,
+                   int64_t stride_x_b, int64_t stride_x_r, int64_t stride_x_h,
+                   int64_t stride_o_b, int64_t stride_o_r, int64_t stride_o_h,
+                   int dtype, void* stream);
 
 /* Absorb the query into the per-kv-head factor: qt[b, h, rho] = sum_d q[b, h, d] * B[b, h / G, rho, d]
  * as a 16-bit high part `qt_hi` and (optional, may be NULL) residual `qt_lo` so that hi + lo carries

@@ -12,11 +12,12 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("XKV_HIP_LIB", os.path.join(_HERE, "libxkv_hip.so"))  # override: another build of the same ABI
 
 XKV_F16, XKV_BF16, XKV_F32 = 0, 1, 2
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 EXPORTS = (
     "xkv_abi_version", "xkv_error_string", "xkv_rope_table", "xkv_absorb_q",
     "xkv_blockdiag_q", "xkv_latent_stage1", "xkv_recon_stage1", "xkv_recon_workspace_bytes", "xkv_merge_stage2",
+    "xkv_rope_apply",
 )
 
 
@@ -39,6 +40,9 @@ def _declare(lib):
     lib.xkv_error_string.argtypes = [c_int]
     lib.xkv_rope_table.restype = c_int
     lib.xkv_rope_table.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_void_p]
+    lib.xkv_rope_apply.restype = c_int
+    lib.xkv_rope_apply.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int,
+                                   c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]
     lib.xkv_absorb_q.restype = c_int
     lib.xkv_absorb_q.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                  c_int64, c_int64, c_int64, c_int, c_void_p]

@@ -24,6 +24,34 @@ __global__ void rope_table_kernel(O* __restrict__ sin_out, O* __restrict__ cos_o
 }
 
 // ----------------------------------------------------------------------------------------------
+// Rotate-half RoPE applied to rows x[b, r, h, :] at position (positions ? positions[b] : pos0) + r: one thread per pair
+// (j, j + dim/2), fp32 angle float(pos) * inv_freq[j] and fp32 arithmetic as in the eager form (rope/rope_ref.py:3-20).
+// ----------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void rope_apply_kernel(const T* __restrict__ x, T* __restrict__ out,
+                                                          const float* __restrict__ inv_freq,
+                                                          const int64_t* __restrict__ positions, int64_t pos0, int64_t total,
+                                                          int rows, int heads, int half, int64_t sxb, int64_t sxr, int64_t sxh,
+                                                          int64_t sob, int64_t sor, int64_t soh) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int j = (int)(idx % half);
+  int64_t t = idx / half;
+  const int h = (int)(t % heads);
+  t /= heads;
+  const int r = (int)(t % rows);
+  const int64_t b = t / rows;
+  const int64_t pos = (positions ? positions[b] : pos0) + r;
+  float s, c;
+  sincosf((float)pos * inv_freq[j], &s, &c);
+  const T* xi = x + b * sxb + r * sxr + h * sxh;
+  T* oi = out + b * sob + r * sor + h * soh;
+  const float x0 = (float)xi[j], x1 = (float)xi[j + half];
+  oi[j] = (T)(x0 * c - x1 * s);
+  oi[j + half] = (T)(x1 * c + x0 * s);
+}
+
+// ----------------------------------------------------------------------------------------------
 // qt[b,h,rho] = sum_d q[b,h,d] * B[b,h/G,rho,d]; one workgroup per (kv head, batch), one thread
 // per rho (strided), the G query rows of the kv head held in LDS as fp32.
 // ----------------------------------------------------------------------------------------------
@@ -371,6 +399,33 @@ extern "C" int xkv_rope_table(void* sin_out, void* cos_out, const float* inv_fre
     case XKV_F32: return launch_rope<float>(sin_out, cos_out, inv_freq, seqlen, start, half_dim, st);
     case XKV_F16: return launch_rope<_Float16>(sin_out, cos_out, inv_freq, seqlen, start, half_dim, st);
     case XKV_BF16: return launch_rope<__bf16>(sin_out, cos_out, inv_freq, seqlen, start, half_dim, st);
+    default: return XKV_EDTYPE;
+  }
+}
+
+template <typename T>
+static int launch_rope_apply(const void* x, void* out, const float* inv_freq, const int64_t* positions, int64_t pos0,
+                             int batch, int rows, int heads, int dim, int64_t sxb, int64_t sxr, int64_t sxh, int64_t sob,
+                             int64_t sor, int64_t soh, hipStream_t st) {
+  const int64_t total = (int64_t)batch * rows * heads * (dim / 2);
+  const int64_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffff) return XKV_EUNSUPPORTED;
+  rope_apply_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, st>>>((const T*)x, (T*)out, inv_freq, positions, pos0, total, rows,
+                                                                      heads, dim / 2, sxb, sxr, sxh, sob, sor, soh);
+  return launch_status();
+}
+
+extern "C" int xkv_rope_apply(const void* x, void* out, const float* inv_freq, const int64_t* positions, int64_t pos0,
+                              int batch, int rows, int heads, int dim, int64_t sxb, int64_t sxr, int64_t sxh,
+                              int64_t sob, int64_t sor, int64_t soh, int dtype, void* stream) {
+  if (!x || !out || !inv_freq || batch < 0 || rows < 0 || heads <= 0 || dim <= 0) return XKV_EINVAL;
+  if (dim % 2) return XKV_EUNSUPPORTED;
+  if (batch == 0 || rows == 0) return XKV_OK;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case XKV_F32: return launch_rope_apply<float>(x, out, inv_freq, positions, pos0, batch, rows, heads, dim, sxb, sxr, sxh, sob, sor, soh, st);
+    case XKV_F16: return launch_rope_apply<_Float16>(x, out, inv_freq, positions, pos0, batch, rows, heads, dim, sxb, sxr, sxh, sob, sor, soh, st);
+    case XKV_BF16: return launch_rope_apply<__bf16>(x, out, inv_freq, positions, pos0, batch, rows, heads, dim, sxb, sxr, sxh, sob, sor, soh, st);
     default: return XKV_EDTYPE;
   }
 }

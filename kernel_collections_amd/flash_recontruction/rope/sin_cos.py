@@ -21,3 +21,12 @@ def rotary_sin_cos(seqlen: int, theta: float = 10_000.0, starting_idx: int = 0, 
         with torch.cuda.stream(stream):
             return ops.rope_table(seqlen, theta, starting_idx, dtype, device)
     return ops.rope_table(seqlen, theta, starting_idx, dtype, device)
+
+
+def rotary_apply(x, positions, theta: float = 10_000.0, *, out=None):
+    """Rotate ``x`` to absolute ``positions`` on the device - what a caller of the ``q_pe`` entry points otherwise does
+    in eager torch (reference rope_ref.py:17-20 on the tables of rope_ref.py:3-9).  ``x`` is ``[batch, heads, dim]`` (one
+    position per sequence: the decode query) or ``[batch, rows, heads, dim]`` (row r at ``positions[b] + r``: a tail of new
+    keys); ``positions`` an int or an integer tensor ``[batch]``.  Returns a new tensor (or ``out``; ``out=x`` rotates in
+    place)."""
+    return ops.rope_apply(x, positions, theta, out)

@@ -110,6 +110,33 @@ def rope_table(seqlen: int, theta: float, start: int, dtype, device, half_dim: i
     return sin, cos
 
 
+def rope_apply(x: torch.Tensor, positions, theta: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rotate-half RoPE on the device.  x ``[batch, heads, dim]`` (one row per sequence, e.g. the decode query) or
+    ``[batch, rows, heads, dim]`` (row r of sequence b sits at ``positions[b] + r``); ``positions`` an int or an integer
+    tensor ``[batch]`` (kept on the device: no host synchronisation).  fp32 angles ``float(pos) * inv_freq`` as in the
+    reference's eager form (flash_recontruction/rope/rope_ref.py:3-20); x may be float32, float16 or bfloat16."""
+    _lib.require_gpu(x)
+    assert x.dim() in (3, 4) and x.stride(-1) == 1 and x.shape[-1] % 2 == 0
+    x4 = x.unsqueeze(1) if x.dim() == 3 else x
+    if out is None:
+        out = torch.empty_like(x)
+    assert out.shape == x.shape and out.dtype == x.dtype and out.stride(-1) == 1 and out.device == x.device
+    o4 = out.unsqueeze(1) if out.dim() == 3 else out
+    b, rows, heads, dim = x4.shape
+    pos_t, pos0 = None, 0
+    if torch.is_tensor(positions):
+        assert positions.numel() == b
+        pos_t = positions.to(device=x.device, dtype=torch.int64).contiguous()
+    else:
+        pos0 = int(positions)
+    inv = rope_inv_freq(dim, theta, x.device)
+    check(_lib.lib().xkv_rope_apply(ptr(x4), ptr(o4), ptr(inv), ptr(pos_t), c_int64(pos0), b, rows, heads, dim,
+                                    c_int64(x4.stride(0)), c_int64(x4.stride(1)), c_int64(x4.stride(2)),
+                                    c_int64(o4.stride(0)), c_int64(o4.stride(1)), c_int64(o4.stride(2)),
+                                    dtype_code(x.dtype), stream_ptr(x)), "xkv_rope_apply")
+    return out
+
+
 def absorb_q(q3: torch.Tensor, Bk: torch.Tensor, want_lo: bool = True) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """q3 `[b,Hq,d]`, Bk `[b,Hkv,r,d]` (any batch/head/rank strides) -> q~ hi (and lo) `[b,Hq,r]`."""
     b, hq, d = q3.shape

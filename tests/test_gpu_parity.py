@@ -41,6 +41,36 @@ def test_rope_table(dev, theta, start):
     assert max_abs(sin, osin[:, :64]) < 2e-6 and max_abs(cos, ocos[:, :64]) < 2e-6
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, BF, FP])
+def test_rope_apply(dev, dtype):
+    """Device-side rotation of a decode query (one position per sequence) and of a tail of new keys (consecutive
+    positions) against the oracle's eager rotate-half form on fp32 angles, at positions 0, 4096 and 131071."""
+    from kernel_collections_amd.flash_recontruction.rope.sin_cos import rotary_apply
+    theta, d = 5e5, 128
+    pos = [0, 4096, 131071]
+    q = gen((3, 32, d), dtype=dtype, seed=1)
+    cos, sin = oracle.rope_cos_sin(torch.tensor(pos), d, theta)
+    ref = oracle.apply_rope(q.float(), cos[:, None, :], sin[:, None, :])
+    tol = 2e-6 if dtype == torch.float32 else (2.0 ** -8 if dtype == BF else 2.0 ** -11)   # one rounding of the output type
+    out = rotary_apply(q.to(dev), torch.tensor(pos, device=dev), theta)
+    assert out.dtype == dtype and out.shape == q.shape
+    assert rel_max(out, ref) <= tol
+    assert max_abs(rotary_apply(q[1:2].to(dev), 4096, theta), ref[1:2]) <= tol * ref.abs().max().item()   # integer position
+    # a tail of 70 keys per sequence, starting at 131071 - 69 / 0 / 4096, written in place into a strided view
+    L, hkv = 70, 8
+    K = gen((3, L, hkv, d + 8), dtype=dtype, seed=2)
+    starts = [131071 - (L - 1), 0, 4096]
+    refs = []
+    for i, s0 in enumerate(starts):
+        c, s_ = oracle.rope_cos_sin(torch.arange(s0, s0 + L), d, theta)
+        refs.append(oracle.apply_rope(K[i, :, :, :d].float(), c[:, None, :], s_[:, None, :]))
+    Kd = K.to(dev)
+    view = Kd[..., :d]
+    assert rotary_apply(view, torch.tensor(starts, device=dev), theta, out=view) is view
+    assert rel_max(Kd[..., :d], torch.stack(refs)) <= tol
+    assert torch.equal(Kd[..., d:].cpu(), K[..., d:]), "the padding columns of the strided view are untouched"
+
+
 # ------------------------------------------------------------------------------------ qAB, no PE
 @pytest.mark.parametrize("dtype", [BF, FP])
 @pytest.mark.parametrize("b,hq,hkv,L,r", [(2, 32, 8, 1000, 512), (1, 8, 8, 77, 192), (3, 16, 2, 4133, 256),
