@@ -37,7 +37,8 @@ enum {
   XKV_EINVAL = -1,      /* null pointer / non-positive size */
   XKV_EUNSUPPORTED = -2,/* shape outside the built envelope (see each function) */
   XKV_EALIGN = -3,      /* stride or pointer not 16-byte aligned */
-  XKV_EDTYPE = -4
+  XKV_EDTYPE = -4,
+  XKV_ESCRATCH = -5     /* xkv_recon_stage1_static: needs more than XKV_STATIC_SCRATCH_BYTES */
 };
 
 int xkv_abi_version(void);
@@ -163,6 +164,28 @@ int xkv_recon_stage1(const void* q_pe, xkv_kv_operand kA, const void* kB,
  * operand order: one copy per batch entry, a single copy when stride_kB_b == 0).  0: no fast path for this rank.
  * Passing workspace == NULL (or too few bytes) is valid and selects the generic kernel.  No reference counterpart. */
 int64_t xkv_recon_workspace_bytes(int batch, int hkv, int rank, int64_t stride_kB_b);
+
+/* xkv_recon_stage1 for callers that cannot allocate device memory (code under HIP graph capture, serving loops or
+ * harnesses that forbid hipMalloc): the same arguments without the workspace, the same kernels and results.  The scratch
+ * that the fast paths need (xkv_recon_workspace_bytes(): kB re-packed into MFMA operand order) is a static device array of
+ * XKV_STATIC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process ends; the call allocates and
+ * frees nothing.  A shape that needs more (hkv * rank * 128 * 2 bytes per copy of kB, one copy per batch entry unless
+ * stride_kB_b == 0) returns XKV_ESCRATCH and launches nothing.  Every call on a GPU uses that GPU's one array and
+ * overwrites what the previous call left there: calls on the same GPU must not overlap (two streams, two threads) - they
+ * would race on it; calls in stream order on one stream are safe.  The device current at the call must be the stream's.
+ * No counterpart in the reference, whose wrappers allocate with torch.empty on every call
+ * (flash_recontruction/fused_attention/no_pe/v1.py:434-446). */
+#define XKV_STATIC_SCRATCH_BYTES (4 << 20)
+int xkv_recon_stage1_static(const void* q_pe, xkv_kv_operand kA, const void* kB,
+                            int64_t stride_kB_b, int64_t stride_kB_h, int64_t stride_kB_r,
+                            xkv_kv_operand vA,
+                            float* partial, float* lse,
+                            void* scores_out, int scores_dtype,
+                            const int32_t* num_kv_splits, const int32_t* kv_lens,
+                            int batch, int hq, int hkv, int kv_len, int max_splits,
+                            float sm_scale, int rope, const float* inv_freq, int64_t pos_offset,
+                            const void* sin_cos, int64_t sc_stride_l,
+                            int dtype, void* stream);
 
 /* Stage 2: LSE-weighted merge of the live splits in increasing split id,
  *   out[b,h,:] = sum_i w_i partial[b,h,i,:] / sum_i w_i ,  w_i = exp(lse_i - max lse),

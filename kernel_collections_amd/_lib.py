@@ -17,8 +17,10 @@ ABI_VERSION = 3
 EXPORTS = (
     "xkv_abi_version", "xkv_error_string", "xkv_rope_table", "xkv_absorb_q",
     "xkv_blockdiag_q", "xkv_latent_stage1", "xkv_recon_stage1", "xkv_recon_workspace_bytes", "xkv_merge_stage2",
-    "xkv_rope_apply",
+    "xkv_recon_stage1_static", "xkv_rope_apply",
 )
+STATIC_SCRATCH_BYTES = 4 << 20
+XKV_ESCRATCH = -5
 
 
 class KVOperand(Structure):
@@ -57,6 +59,8 @@ def _declare(lib):
                                      c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_int64,
                                      c_void_p, c_int64, c_void_p, c_int64, c_int, c_void_p]
+    lib.xkv_recon_stage1_static.restype = c_int
+    lib.xkv_recon_stage1_static.argtypes = lib.xkv_recon_stage1.argtypes[:-4] + [c_int, c_void_p]
     lib.xkv_recon_workspace_bytes.restype = c_int64
     lib.xkv_recon_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int64]
     lib.xkv_merge_stage2.restype = c_int

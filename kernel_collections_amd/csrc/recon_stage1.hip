@@ -18,6 +18,7 @@
 // range-reduced sincosf every 32 tiles and advanced by a constant rotation in between.
 #include "xkv_common.h"
 #include "recon_fast.h"
+#include <mutex>
 
 namespace xkv {
 
@@ -433,4 +434,54 @@ extern "C" int xkv_recon_stage1(const void* q_pe, xkv_kv_operand kA, const void*
     if (rc != DUO_NOT_MINE) return rc;
   }
   return dtype == XKV_BF16 ? dispatch_recon<__bf16>(p, batch, vshared, st) : dispatch_recon<_Float16>(p, batch, vshared, st);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// The same stage 1 for callers that cannot allocate: the packed copy of kB lives in a file-scope device array instead of
+// a caller workspace.  Every GPU holds its own copy of the array at its own address; the address is looked up once per
+// device (first call with that device current) and kept.  The array's NAME is only a host-side handle for that lookup:
+// kernels and copies always get the looked-up pointer.
+// ---------------------------------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[XKV_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[MAX_DEVICES];   // device address of `scratch` on each GPU, NULL until looked up
+
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= MAX_DEVICES) return XKV_EUNSUPPORTED;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!ptr) return (int)hipErrorInvalidSymbol;
+    scratch_ptr[dev] = ptr;
+  }
+  *out = scratch_ptr[dev];
+  return XKV_OK;
+}
+}  // namespace
+
+extern "C" int xkv_recon_stage1_static(const void* q_pe, xkv_kv_operand kA, const void* kB, int64_t sBb, int64_t sBh,
+                                       int64_t sBr, xkv_kv_operand vA, float* partial, float* lse, void* scores_out,
+                                       int scores_dtype, const int32_t* num_kv_splits, const int32_t* kv_lens,
+                                       int batch, int hq, int hkv, int kv_len, int max_splits, float sm_scale, int rope,
+                                       const float* inv_freq, int64_t pos_offset, const void* sin_cos,
+                                       int64_t sc_stride_l, int dtype, void* stream) {
+  if (batch <= 0 || hkv <= 0) return XKV_EINVAL;
+  const int64_t need = xkv_recon_workspace_bytes(batch, hkv, kA.dim, sBb);
+  if (need > (int64_t)XKV_STATIC_SCRATCH_BYTES) return XKV_ESCRATCH;   // nothing is launched
+  void* ws = nullptr;
+  if (need > 0) {
+    const int rc = static_scratch(&ws);
+    if (rc != XKV_OK) return rc;
+  }
+  return xkv_recon_stage1(q_pe, kA, kB, sBb, sBh, sBr, vA, partial, lse, scores_out, scores_dtype, num_kv_splits, kv_lens,
+                          batch, hq, hkv, kv_len, max_splits, sm_scale, rope, inv_freq, pos_offset, sin_cos, sc_stride_l,
+                          ws, need, dtype, stream);
 }

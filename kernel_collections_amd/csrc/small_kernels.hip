@@ -386,6 +386,7 @@ extern "C" const char* xkv_error_string(int code) {
     case XKV_EUNSUPPORTED: return "shape outside the built envelope";
     case XKV_EALIGN: return "pointer or stride not 16-byte aligned";
     case XKV_EDTYPE: return "unsupported dtype code";
+    case XKV_ESCRATCH: return "the call needs more scratch than the library's static device array holds";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown xkv error";
   }
 }

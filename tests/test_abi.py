@@ -46,6 +46,12 @@ def test_argument_errors_are_reported_before_any_launch():
     assert rc == -2
     with pytest.raises(RuntimeError, match="envelope"):
         _lib.check(rc, "xkv_latent_stage1")
+    # the static-scratch variant refuses a shape whose packed factors exceed its array (8 x 1 MiB here), before any HIP call
+    big = _lib.KVOperand(ctypes.c_void_p(16), 512 * 64, 512, 0, 512)
+    rc = L.xkv_recon_stage1_static(ctypes.c_void_p(16), big, ctypes.c_void_p(16), 8 * 512 * 128, 512 * 128, 128, big,
+                                   ctypes.c_void_p(16), ctypes.c_void_p(16), null, 0, ns, null, 8, 32, 8, 64, 1, 1.0, 1,
+                                   ctypes.c_void_p(16), 0, null, 0, _lib.XKV_BF16, null)
+    assert rc == _lib.XKV_ESCRATCH and b"static device array" in L.xkv_error_string(rc)
 
 
 def test_python_surface_matches_reference_names_and_argument_order():
