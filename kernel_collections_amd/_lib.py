@@ -17,7 +17,7 @@ ABI_VERSION = 3
 EXPORTS = (
     "xkv_abi_version", "xkv_error_string", "xkv_rope_table", "xkv_absorb_q",
     "xkv_blockdiag_q", "xkv_latent_stage1", "xkv_recon_stage1", "xkv_recon_workspace_bytes", "xkv_merge_stage2",
-    "xkv_recon_stage1_static", "xkv_rope_apply",
+    "xkv_recon_stage1_static", "xkv_rope_apply", "xkv_ceiling_mfma", "xkv_ceiling_stream",
 )
 STATIC_SCRATCH_BYTES = 4 << 20
 XKV_ESCRATCH = -5
@@ -45,6 +45,10 @@ def _declare(lib):
     lib.xkv_rope_apply.restype = c_int
     lib.xkv_rope_apply.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int,
                                    c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]
+    lib.xkv_ceiling_mfma.restype = c_int
+    lib.xkv_ceiling_mfma.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p]
+    lib.xkv_ceiling_stream.restype = c_int
+    lib.xkv_ceiling_stream.argtypes = [c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p]
     lib.xkv_absorb_q.restype = c_int
     lib.xkv_absorb_q.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                  c_int64, c_int64, c_int64, c_int, c_void_p]

@@ -4,7 +4,10 @@ tile loaded once (the reference reuses it through ``tl.trans``, stage1.py:150)."
 from kernel_collections_amd import ops
 
 
-def decoding_stage1(q_nope, q_rope, kv_nope, k_rope, attn_out, attn_lse, num_kv_splits, max_kv_splits, sm_scale):
+def decoding_stage1(q_nope, q_rope, kv_nope, k_rope, attn_out, attn_lse, num_kv_splits, max_kv_splits, sm_scale, *,
+                    q_nope_lo=None):
+    """``q_nope_lo`` (keyword-only, not in the reference): residual of an absorbed query kept as a high + low 16-bit pair
+    (``ops.absorb_q``); its dot with the latent is added to the scores."""
     batch, head_num, dmodel = q_nope.shape
     assert kv_nope.dim() == 4 and k_rope.dim() == 4
     n_kv = kv_nope.shape[2]
@@ -22,5 +25,5 @@ def decoding_stage1(q_nope, q_rope, kv_nope, k_rope, attn_out, attn_lse, num_kv_
     splits = ops.as_int32_dev(num_kv_splits, batch, q_nope.device)
     C = (kv_nope, kv_nope.stride(0), kv_nope.stride(1), sh_c, dmodel)
     R = (k_rope, k_rope.stride(0), k_rope.stride(1), sh_r, k_rope.shape[-1])
-    ops.latent_stage1(ops._q3(q_nope), None, ops._q3(q_rope), C, R, C, attn_out, attn_lse, None, splits, None,
+    ops.latent_stage1(ops._q3(q_nope), None if q_nope_lo is None else ops._q3(q_nope_lo), ops._q3(q_rope), C, R, C, attn_out, attn_lse, None, splits, None,
                       batch, head_num, groups, kv_len, int(max_kv_splits), float(sm_scale))

@@ -14,7 +14,21 @@ from . import _lib
 from ._lib import check, dtype_code, kv_operand, ptr, q_operand, stream_ptr
 
 _16BIT = (torch.float16, torch.bfloat16)
-_NUM_CU = 256  # MI355X
+_num_cu_cache = {}
+
+
+def num_cus(device=None) -> int:
+    """Compute units of the device, read from its properties (256 on an MI355X)."""
+    if not torch.cuda.is_available():
+        return 256   # planning a split count off the device (CPU-side tests): the MI355X figure
+    idx = torch.cuda.current_device() if device is None else torch.device(device).index
+    if idx is None:
+        idx = torch.cuda.current_device()
+    n = _num_cu_cache.get(idx)
+    if n is None:
+        n = _num_cu_cache[idx] = int(torch.cuda.get_device_properties(idx).multi_processor_count)
+    return n
+
 USE_RECON_WORKSPACE = True  # False: never hand xkv_recon_stage1 a workspace (it then takes its generic kernel)
 
 
@@ -55,7 +69,7 @@ def uniform_splits(batch: int, n: int, device) -> torch.Tensor:
 def occupancy_splits(batch: int, groups: int, kv_len: int, tile: int = 64, waves: int = 2) -> int:
     """Number of KV splits that gives about `waves` workgroups per CU without making a split
     shorter than 4 tiles."""
-    want = _cdiv(waves * _NUM_CU, max(1, batch * groups))
+    want = _cdiv(waves * num_cus(), max(1, batch * groups))
     cap = max(1, kv_len // (4 * tile))
     return max(1, min(want, cap))
 

@@ -4,8 +4,14 @@ the uncompressed flash decode, and its distance from the eager result.
 
     python -m kernel_collections_amd.profiling --kv_len 131072 --k_rank 384 --v_rank 512 [--batch 1] [--dtype bf16]
 
-Same flags as the reference script (:511-517: --num_heads --num_kv_heads --head_dim --kv_len --k_rank --v_rank);
---profile prints the per-kernel table of torch.profiler for one pass over the variants instead of writing a trace.
+Same flags as the reference script (:511-517: --num_heads --num_kv_heads --head_dim --kv_len --k_rank --v_rank).
+--profile runs one pass over the variants under torch.profiler, one ``record_function`` range per variant, prints the
+per-kernel table and exports the chrome trace (``--trace_path``, default ./xkv_profile_trace.json), as the reference's
+profiling pass does (:118-211).
+--sweep is the key-reconstruction sweep of the reference's test_qAB_rope.py:85-167 / test_fused_key_reconstruction.py:94-100:
+kv_len 2^14 .. 2^17 at batch 1, rank --k_rank (192 there), fp16 by default; per kv_len the plain q.K^T of torch and the
+four qAB-with-RoPE entry points (v2 on a precomputed sin/cos table), each as median / 20 % / 80 % quantile over --repeat
+timed calls after --warmup (the reference: 100 after 25).
 The eager and SDPA rows are torch on the same device (comparators, as in the reference); every other row runs the
 HIP kernels of this package."""
 from __future__ import annotations
@@ -31,6 +37,57 @@ def _time(fn, warmup=5, repeat=20):
     en.record()
     torch.cuda.synchronize()
     return st.elapsed_time(en) / repeat
+
+
+def _quantiles(fn, warmup=25, repeat=100):
+    """(median, 20 %, 80 %) in ms over `repeat` calls timed one by one with HIP events (what triton.testing.do_bench
+    returns for quantiles=[0.5, 0.2, 0.8], test_qAB_rope.py:136-163)."""
+    for _ in range(warmup):
+        fn()
+    st = [torch.cuda.Event(enable_timing=True) for _ in range(repeat)]
+    en = [torch.cuda.Event(enable_timing=True) for _ in range(repeat)]
+    torch.cuda.synchronize()
+    for i in range(repeat):
+        st[i].record()
+        fn()
+        en[i].record()
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in zip(st, en))
+    pick = lambda f: ts[min(repeat - 1, int(f * repeat))]
+    return pick(0.5), pick(0.2), pick(0.8)
+
+
+def sweep(args):
+    """kv_len sweep of the RoPE key-reconstruction scores; returns [(kv_len, {operation: (median, p20, p80)})]."""
+    from kernel_collections_amd.flash_recontruction.rope.sin_cos import rotary_sin_cos
+    dev = torch.device("cuda:0")
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float16
+    hq, hkv, d, r, theta = args.num_heads, args.num_kv_heads, args.head_dim, args.k_rank, 1e7
+    g = torch.Generator(device=dev).manual_seed(0)
+    rnd = lambda shape: torch.randn(shape, device=dev, dtype=torch.float32, generator=g).to(dtype)
+    rows = []
+    for e in range(args.sweep_min, args.sweep_max + 1):
+        L = 2 ** e
+        q, K = rnd((1, hq, 1, d)), rnd((1, hkv, L, d))
+        Ak, Bk = rnd((1, L, r)), rnd((1, hkv, r, d))
+        sin, cos = rotary_sin_cos(L, theta, 0, dtype=dtype, device=dev)
+        sin_cos = torch.cat((sin, cos), dim=-1)
+        qg = q.reshape(1, hkv, hq // hkv, d)
+        ops_ = {
+            "qK (torch)": lambda: torch.matmul(qg, K.transpose(-1, -2)),
+            "qAB_v1": lambda: fr.qAB_rope_v1(q, Ak, Bk, theta),
+            "qAB_v2 (table)": lambda: fr.qAB_rope_v2(q, Ak, Bk, sin_cos),
+            "qAB_v3": lambda: fr.qAB_rope_v3(q, Ak, Bk, theta),
+            "qAB_v4": lambda: fr.qAB_rope_v4(q, Ak, Bk, theta),
+        }
+        rows.append((L, {name: _quantiles(fn, args.warmup, args.repeat) for name, fn in ops_.items()}))
+    names = list(rows[0][1])
+    print("\n=== qK vs qAB with RoPE: batch 1, %d q / %d kv heads, head_dim %d, rank %d, %s; ms as median [20 %% .. 80 %%] ==="
+          % (hq, hkv, d, r, args.dtype))
+    print("%10s " % "kv_len" + " ".join("%26s" % n for n in names))
+    for L, res in rows:
+        print("%10d " % L + " ".join("%10.4f [%6.4f..%6.4f]" % res[n] for n in names))
+    return rows
 
 
 def eager_attention(q, K, V, scale):
@@ -88,12 +145,18 @@ def run(args):
     variants = build_variants(args.batch, args.num_heads, args.num_kv_heads, args.head_dim, args.kv_len, args.k_rank,
                               args.v_rank, dtype, dev)
     if args.profile:
-        from torch.profiler import ProfilerActivity, profile
+        from torch.profiler import ProfilerActivity, profile, record_function
+        for _, fn, _ in variants:   # first calls (module load, allocator growth) stay out of the trace
+            fn()
+        torch.cuda.synchronize()
         with profile(activities=[ProfilerActivity.CPU, ProfilerActivity.CUDA]) as prof:
-            for _, fn, _ in variants:
-                fn()
-            torch.cuda.synchronize()
+            for name, fn, _ in variants:
+                with record_function(name):
+                    fn()
+                torch.cuda.synchronize()
         print(prof.key_averages().table(sort_by="cuda_time_total", row_limit=20))
+        prof.export_chrome_trace(args.trace_path)
+        print("chrome trace written to %s" % args.trace_path)
         return []
     ref = variants[0][1]().float()
     rows = []
@@ -127,8 +190,13 @@ def main(argv=None):
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"])
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--repeat", type=int, default=20)
-    ap.add_argument("--profile", action="store_true")
-    return run(ap.parse_args(argv))
+    ap.add_argument("--profile", action="store_true", help="one profiled pass over the variants; writes a chrome trace")
+    ap.add_argument("--trace_path", default="xkv_profile_trace.json")
+    ap.add_argument("--sweep", action="store_true", help="kv_len sweep of the qAB-with-RoPE entry points (rank = --k_rank)")
+    ap.add_argument("--sweep_min", type=int, default=14, help="log2 of the first kv_len of the sweep")
+    ap.add_argument("--sweep_max", type=int, default=17, help="log2 of the last kv_len of the sweep")
+    args = ap.parse_args(argv)
+    return sweep(args) if args.sweep else run(args)
 
 
 if __name__ == "__main__":

@@ -159,3 +159,91 @@ def test_refined_splits_follow_the_lengths_and_their_updates():
     assert out4.tolist() == [7, 1, 1, 2, 26]
     uni, Su = gqa._refine_splits(torch.full((3,), 2, dtype=torch.int32), None, 3, 5000, 2, 2048, lens.device)
     assert uni.tolist() == [3, 3, 3] and Su == 3
+
+
+REFERENCE_IMPORTS = """
+from flash_recontruction import qAB_no_pe_v1, qAB_no_pe_v2, qAB_no_pe_ref, qAB_rope_v1, qAB_rope_v2, qAB_rope_v3, qAB_rope_v4
+from flash_recontruction import gqa_xKV_no_pe_ref, gqa_xKV_no_pe_k_only_ref, gqa_xKV_no_pe_k_only, gqa_xKV_no_pe, gqa_xKV_no_pe_v2
+from flash_recontruction.rope.sin_cos import rotary_sin_cos
+from flash_recontruction.rope.rope_ref import LlamaRotaryEmbedding, rotate_half, apply_rotary_pos_emb_pytorch
+from flash_decoding.gqa import decode_attention_fwd
+from flash_decoding.mla import decode_attention_fwd, decode_attention_reference
+from flash_decoding.mla2 import mla_decode_attention_fwd, mla_decode_attention_fwd_ref, mla_decode_attention_xKV
+from flash_decoding.deepseek_mla import mla_decode_attention_fwd, mla_decode_attention_fwd_pd_sep, mla_decode_attention_fwd_pd_sep_xKV
+"""
+
+
+def _doc_python_blocks():
+    """Every fenced python block of the markdown notes at the repository root."""
+    out = []
+    for name in sorted(os.listdir(ROOT)):
+        if name.endswith(".md"):
+            text = open(os.path.join(ROOT, name)).read()
+            out += [(name, m.group(1)) for m in re.finditer(r"```python\n(.*?)```", text, flags=re.S)]
+    return out
+
+
+def test_install_aliases_binds_the_reference_module_names():
+    """After install_aliases() code written against the reference imports unchanged: every name the reference's scripts
+    import (test_gqa_xKV.py:1-10, test_qAB_rope.py:1-8, test_triton_gqa.py:1, test_triton_mla.py:1,
+    test_mla_decoding_new.py:1, test_mla_decoding_new2.py:3, test_cos_sin.py:1-3), and the import block the notes print."""
+    import sys
+    import kernel_collections_amd
+    saved = {k: sys.modules.get(k) for k in ("flash_recontruction", "flash_decoding")}
+    try:
+        kernel_collections_amd.install_aliases()
+        exec(REFERENCE_IMPORTS, {})
+        blocks = [code for _, code in _doc_python_blocks() if "install_aliases()" in code]
+        assert blocks, "the notes show the import route"
+        for code in blocks:
+            exec(code, {})
+        import flash_recontruction
+        assert flash_recontruction is sys.modules["kernel_collections_amd.flash_recontruction"]
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                sys.modules.pop(k, None)
+            else:
+                sys.modules[k] = v
+
+
+def _load_route_b_stub(monkeypatch):
+    import importlib.util
+    from kernel_collections_amd import _lib
+    monkeypatch.setenv("XKV_HIP_LIB", _lib.LIB_PATH)
+    spec = importlib.util.spec_from_file_location("route_b_stub", os.path.join(ROOT, "tests", "route_b_stub.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)      # loads the library, declares the prototype, checks the ABI version
+    return mod
+
+
+def test_ctypes_stub_of_the_notes_loads_and_is_the_printed_one(monkeypatch):
+    mod = _load_route_b_stub(monkeypatch)
+    assert callable(mod.qAB)
+    printed = [code for _, code in _doc_python_blocks() if "xkv_recon_stage1.argtypes" in code]
+    assert len(printed) == 1
+    body = open(os.path.join(ROOT, "tests", "route_b_stub.py")).read()
+    assert body.endswith(printed[0]), "tests/route_b_stub.py must stay word for word what the notes print"
+    from kernel_collections_amd import _lib
+    assert mod._xkv.xkv_recon_stage1.argtypes[1]._fields_ == _lib.KVOperand._fields_
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_ctypes_stub_of_the_notes_computes_qab_rope(monkeypatch, dtype):
+    """The stub binds nothing but ctypes and torch; its qAB must give the reference's RoPE scores."""
+    import oracle
+    mod = _load_route_b_stub(monkeypatch)
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(5)
+    b, hq, hkv, L, r, d, theta = 2, 32, 8, 700, 512, 128, 1e7
+    q = (torch.randn(b, hq, 1, d, generator=g) * 0.5).to(dtype)
+    A = torch.randn(b, L, r, generator=g).to(dtype)
+    B = (torch.randn(b, hkv, r, d, generator=g) * r ** -0.5).to(dtype)
+    cos, sin = oracle.rope_cos_sin(torch.arange(L), d, theta)
+    ref = oracle.qab_rope(q.float(), A.float(), B.float(), cos, sin)
+    out = mod.qAB(q.to(dev), A.to(dev), B.to(dev), theta)
+    torch.cuda.synchronize()
+    assert out.shape == (b, hq, 1, L) and out.dtype == dtype
+    err = (out.float().cpu() - ref).abs().max().item() / ref.abs().max().item()
+    assert err <= 1e-2, err

@@ -1,0 +1,211 @@
+"""GPU parity at the shapes the benchmark configurations and the reference's own scripts run - full size, not shortened.
+
+Inputs this large are drawn on the device (seeded); the sequences the oracle checks are copied to the CPU, so both sides
+still see identical 16-bit values.  What the oracle cannot cover whole is covered by properties that do not depend on the
+size: every sequence of a ragged batch equals its own batch-1 call, NaN poison past each length is never read, and the
+result does not depend on how the sequence was split.
+"""
+import math
+
+import pytest
+import torch
+
+import oracle
+from util import OUT_ATOL, check_out, check_scores, f32, max_abs
+
+pytestmark = pytest.mark.gpu
+
+import kernel_collections_amd.flash_recontruction as fr  # noqa: E402
+from kernel_collections_amd import ops  # noqa: E402
+from kernel_collections_amd.flash_decoding import gqa, mla, mla2  # noqa: E402
+
+BF, FP = torch.bfloat16, torch.float16
+
+
+def randn_dev(shape, std, dev, dtype, seed):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    out = torch.empty(shape, dtype=dtype, device=dev)
+    flat = out.view(-1)
+    step = 1 << 28   # draw in fp32 slabs of 1 GiB
+    for i in range(0, flat.numel(), step):
+        n = min(step, flat.numel() - i)
+        flat[i:i + n] = (torch.randn(n, device=dev, dtype=torch.float32, generator=g) * std).to(dtype)
+    return out
+
+
+def splits_t(vals, dev):
+    return torch.tensor(vals, dtype=torch.int32, device=dev)
+
+
+def config4_lengths(batch=32, lo=1024, hi=131072, seed=0):
+    """The ragged batch of target configuration 4: lengths log-uniform in [1024, 131072] from a seeded CPU generator."""
+    g = torch.Generator().manual_seed(seed)
+    u = torch.rand(batch, generator=g)
+    return torch.floor(torch.exp(math.log(lo) + u * (math.log(hi) - math.log(lo)))).to(torch.int64).tolist()
+
+
+# ------------------------------------------------------------------------------------ long splits of a ragged batch
+@pytest.mark.parametrize("dtype", [BF, FP])
+def test_ragged_4096_token_splits_with_long_sequences(dev, dtype, monkeypatch):
+    """Per-sequence lengths with 4096-token splits and sequences of 16K+ tokens: the shape at which the two GQA wrappers
+    give long splits to several workgroups.  Against the oracle on every sequence, with NaN poison past each length, and
+    against the same calls with the caller's splits taken as they are."""
+    b, hq, hkv, d, rv, split = 4, 32, 8, 128, 512, 4096
+    lens = [20000, 5000, 1500, 16384 + 77]
+    ns = [-(-n // split) for n in lens]
+    S, Lmax = max(ns), max(lens)
+    scale = d ** -0.5
+    q = randn_dev((b, hq, d), 1.0, dev, dtype, 1)
+    K, V = randn_dev((b, Lmax, hkv, d), 1.0, dev, dtype, 2), randn_dev((b, Lmax, hkv, d), 1.0, dev, dtype, 3)
+    vA, vB = randn_dev((b, Lmax, rv), 1.0, dev, dtype, 4), randn_dev((b, hkv, rv, d), rv ** -0.5, dev, dtype, 5)
+    qc, Kc, Vc, vAc, vBc = (t.cpu() for t in (q, K, V, vA, vB))
+    for i, n in enumerate(lens):
+        K[i, n:] = float("nan"); V[i, n:] = float("nan"); vA[i, n:] = float("nan")
+    ref = oracle.ragged_apply(oracle.gqa_plain, lens, f32(qc, Kc, Vc), (None, 1, 1), sm_scale=scale)
+    ref_v = oracle.ragged_apply(
+        lambda q_, K_, vA_, vB_: oracle.gqa_v_only(q_.unsqueeze(2), K_.transpose(1, 2), vA_, vB_, sm_scale=scale)[:, :, 0],
+        lens, f32(qc, Kc, vAc, vBc), (None, 1, 1, None))
+    kl, nst = splits_t(lens, dev), splits_t(ns, dev)
+    outs = {}
+    for tokens in ("default", 0):
+        if tokens == 0:
+            monkeypatch.setattr(gqa, "REFINE_TOKENS", 0)
+            monkeypatch.setattr(gqa, "REFINE_TOKENS_WIDE", 0)
+        o = torch.zeros_like(q)
+        gqa.decode_attention_fwd(q, K, V, o, nst, S, scale, kv_lens=kl)
+        check_out(o, ref, f"ragged plain, long splits ({tokens})")
+        o2 = torch.zeros_like(q)
+        gqa.decode_attention_fwd_v_factorized(q, K, vA, vB, o2, nst, S, scale, kv_lens=kl)
+        check_out(o2, ref_v, f"ragged V-factorised, long splits ({tokens})")
+        outs[tokens] = (o, o2)
+    assert max_abs(outs["default"][0], outs[0][0]) < 4e-3 and max_abs(outs["default"][1], outs[0][1]) < 4e-3, \
+        "splitting finer must not change the result beyond rounding"
+
+
+# ------------------------------------------------------------------------------------ configuration 4, full size
+@pytest.mark.parametrize("vfact", [False, True], ids=["plain", "v_factorised"])
+def test_config4_full_size(dev, vfact):
+    """Target configuration 4 as configured: batch 32, lengths log-uniform in [1024, 131072], 32 q / 8 kv heads, d 128,
+    4096-token splits, bf16 (K buffer of more than 2^31 elements)."""
+    B, hq, hkv, d, rv, split = 32, 32, 8, 128, 512, 4096
+    lens = config4_lengths(B)
+    Lmax = max(lens)
+    ns = [-(-n // split) for n in lens]
+    S = max(ns)
+    scale = d ** -0.5
+    q = randn_dev((B, hq, d), 1.0, dev, BF, 1)
+    K = randn_dev((B, Lmax, hkv, d), 1.0, dev, BF, 2)
+    assert K.numel() > 2 ** 31
+    if vfact:
+        vA, vB = randn_dev((B, Lmax, rv), 1.0, dev, BF, 3), randn_dev((B, hkv, rv, d), rv ** -0.5, dev, BF, 4)
+    else:
+        V = randn_dev((B, Lmax, hkv, d), 1.0, dev, BF, 3)
+    order = sorted(range(B), key=lambda i: lens[i])
+    picks = [order[0], order[B // 3], order[2 * B // 3], order[-1]]     # shortest, two middle, longest
+    refs = {}
+    for i in picks:
+        n = lens[i]
+        if vfact:
+            refs[i] = oracle.gqa_v_only(q[i:i + 1].cpu().float().unsqueeze(2), K[i:i + 1, :n].cpu().float().transpose(1, 2),
+                                        vA[i:i + 1, :n].cpu().float(), vB[i:i + 1].cpu().float(), sm_scale=scale)[:, :, 0]
+        else:
+            refs[i] = oracle.gqa_plain(q[i:i + 1].cpu().float(), K[i:i + 1, :n].cpu().float(), V[i:i + 1, :n].cpu().float(), scale)
+    for i, n in enumerate(lens):      # poison everything past each sequence's end
+        K[i, n:] = float("nan")
+        if vfact:
+            vA[i, n:] = float("nan")
+        else:
+            V[i, n:] = float("nan")
+    kl, nst = splits_t(lens, dev), splits_t(ns, dev)
+    o = torch.zeros_like(q)
+    if vfact:
+        gqa.decode_attention_fwd_v_factorized(q, K, vA, vB, o, nst, S, scale, kv_lens=kl)
+    else:
+        gqa.decode_attention_fwd(q, K, V, o, nst, S, scale, kv_lens=kl)
+    assert torch.isfinite(o.float()).all()
+    for i in picks:
+        check_out(o[i:i + 1], refs[i], f"config 4, sequence {i} ({lens[i]} tokens)")
+    # every sequence equals its own batch-1 call on its own tokens
+    worst = 0.0
+    for i, n in enumerate(lens):
+        oi = torch.zeros_like(q[i:i + 1])
+        one = splits_t([ns[i]], dev)
+        if vfact:
+            gqa.decode_attention_fwd_v_factorized(q[i:i + 1], K[i:i + 1, :n], vA[i:i + 1, :n], vB[i:i + 1], oi, one, ns[i], scale)
+        else:
+            gqa.decode_attention_fwd(q[i:i + 1], K[i:i + 1, :n], V[i:i + 1, :n], oi, one, ns[i], scale)
+        worst = max(worst, max_abs(oi, o[i:i + 1]))
+    assert worst < 4e-3, f"a sequence of the ragged batch differs from its own batch-1 call by {worst:.3e}"
+
+
+# ------------------------------------------------------------------------------------ the reference scripts' long shapes
+def test_gqa_262144_tokens_128_splits(dev):
+    """test_triton_gqa.py:31-44,72-73 of the reference: batch 1, 32 q / 8 kv heads, d 128, 262144 tokens, 128 splits, fp16
+    N(0,1) inputs at sm_scale 1.0 (logit sigma 11)."""
+    b, hq, hkv, d, L, S = 1, 32, 8, 128, 256 * 1024, 128
+    q, K, V = randn_dev((b, hq, d), 1.0, dev, FP, 1), randn_dev((b, L, hkv, d), 1.0, dev, FP, 2), randn_dev((b, L, hkv, d), 1.0, dev, FP, 3)
+    ref = oracle.gqa_plain(*f32(q.cpu(), K.cpu(), V.cpu()), 1.0)
+    o = torch.zeros_like(q)
+    gqa.decode_attention_fwd(q, K, V, o, splits_t([S], dev), S, 1.0)
+    check_out(o, ref, "gqa 262144 / 128 splits")
+
+
+def test_mla_131328_tokens_head_dim_384(dev):
+    """test_triton_mla.py:8-27,60-67: batch 1, 32 heads on one kv head, head_dim 384, 2048*64+256 tokens (not a multiple of
+    the split), fp16 N(0,1) at sm_scale 1.0."""
+    b, H, dk, L = 1, 32, 384, 2048 * 64 + 256
+    q, K, V = randn_dev((b, H, dk), 1.0, dev, FP, 1), randn_dev((b, L, 1, dk), 1.0, dev, FP, 2), randn_dev((b, L, 1, dk), 1.0, dev, FP, 3)
+    ref = oracle.gqa_plain(*f32(q.cpu(), K.cpu(), V.cpu()), 1.0)
+    o = torch.zeros_like(q)
+    assert mla.decode_attention_fwd(q, K, V, o, 1.0, logit_cap=0.0) is None
+    check_out(o, ref, "mla.py 131328 tokens")
+
+
+def test_mla2_batch4_65536_tokens(dev):
+    """test_mla_decoding_new2.py:7-60: batch 4, 16 heads, latent 512 = kv_A (rank 256) @ kv_B, rope 64, 65536 tokens, fp16
+    inputs drawn as randn / 3 at sm_scale 1.0; both the plain-latent and the factorised-latent entry points."""
+    b, H, c, e, r, L = 4, 16, 512, 64, 256, 64 * 1024
+    qn, qr = randn_dev((b, H, c), 1 / 3, dev, FP, 1), randn_dev((b, H, e), 1 / 3, dev, FP, 2)
+    kvA, kvB = randn_dev((b, L, 1, r), 1 / 3, dev, FP, 3), randn_dev((b, 1, r, c), 1 / 3, dev, FP, 4)
+    kpe = randn_dev((b, L, 1, e), 1 / 3, dev, FP, 5)
+    ckv = torch.matmul(kvA.transpose(1, 2), kvB).transpose(1, 2).contiguous()      # as the script builds it (fp16)
+    out = mla2.mla_decode_attention_fwd(qn, qr, ckv, kpe, 1.0)
+    out_x = mla2.mla_decode_attention_xKV(qn, qr, kvA, kvB, kpe, 1.0)
+    for i in (0, 3):
+        s = slice(i, i + 1)
+        ref = oracle.mla_ref(*f32(qn[s].cpu(), qr[s].cpu(), ckv[s].cpu(), kpe[s].cpu()), 1.0)
+        check_out(out[s], ref, f"mla2, sequence {i}")
+        ref_x = oracle.mla_xkv_ref(*f32(qn[s].cpu(), qr[s].cpu(), kvA[s].cpu(), kvB[s].cpu(), kpe[s].cpu()), 1.0)
+        check_out(out_x[s], ref_x, f"mla2 xKV, sequence {i}")
+
+
+# ------------------------------------------------------------------------------------ configurations 2 and 5, full size
+def test_config2_full_size(dev):
+    """Target configuration 2: batch 8, 32 q / 8 kv heads, d 128, 16384 tokens, rank 512, one B(512 x 1024) for the batch
+    (stride-0 view), bf16 in, fp32 scores out scaled by 1/sqrt(128)."""
+    B, hq, hkv, d, L, r = 8, 32, 8, 128, 16384, 512
+    q, A = randn_dev((B, hq, 1, d), 1.0, dev, BF, 1), randn_dev((B, L, r), 1.0, dev, BF, 2)
+    Bm = randn_dev((r, hkv * d), r ** -0.5, dev, BF, 3)
+    Bv = Bm.view(r, hkv, d).permute(1, 0, 2).unsqueeze(0).expand(B, hkv, r, d)
+    scale = d ** -0.5
+    out = fr.qAB_no_pe_v1(q, A, Bv, sm_scale=scale, out_dtype=torch.float32)
+    assert out.shape == (B, hq, 1, L) and out.dtype == torch.float32
+    ref = oracle.qab_nope(*f32(q.cpu(), A.cpu(), Bv.cpu())) * scale
+    er = check_scores(out, ref, "config 2")
+    assert er < 2e-3
+
+
+def test_config5_full_size(dev):
+    """Target configuration 5: batch 64, 16 heads, latent 512 + rope 64, 8192 tokens, bf16, scale 1/sqrt(192); the oracle on
+    the first and the last sequence, batch-1 equality for four more."""
+    B, H, L, c, e = 64, 16, 8192, 512, 64
+    ckv, kpe = randn_dev((B, L, 1, c), 1.0, dev, BF, 1), randn_dev((B, L, 1, e), 1.0, dev, BF, 2)
+    qn, qr = randn_dev((B, H, c), 0.3, dev, BF, 3), randn_dev((B, H, e), 1.0, dev, BF, 4)
+    scale = 1 / math.sqrt(192)
+    out = mla2.mla_decode_attention_fwd(qn, qr, ckv, kpe, scale)
+    for i in (0, B - 1):
+        s = slice(i, i + 1)
+        check_out(out[s], oracle.mla_ref(*f32(qn[s].cpu(), qr[s].cpu(), ckv[s].cpu(), kpe[s].cpu()), scale), f"config 5, sequence {i}")
+    for i in (1, 17, 40, 62):
+        s = slice(i, i + 1)
+        assert max_abs(mla2.mla_decode_attention_fwd(qn[s], qr[s], ckv[s], kpe[s], scale), out[s]) < 4e-3

@@ -105,3 +105,22 @@ def test_profiling_cli_runs_and_agrees(dev, capsys):
     assert len(rows) == 8 and "Fused xKV v2" in capsys.readouterr().out
     for name, t, err in rows:
         assert t > 0 and (math.isnan(err) or err < 3e-2), (name, err)
+
+
+def test_profiling_cli_sweep_and_trace(dev, capsys, tmp_path):
+    """--sweep prints median / 20 % / 80 % per kv_len and entry point; --profile leaves a chrome trace with one range per variant."""
+    import json
+    from kernel_collections_amd import profiling
+    rows = profiling.main(["--sweep", "--sweep_min", "10", "--sweep_max", "11", "--k_rank", "192", "--dtype", "fp16", "--warmup", "1",
+                           "--repeat", "5"])
+    assert [L for L, _ in rows] == [1024, 2048]
+    for _, res in rows:
+        assert set(res) == {"qK (torch)", "qAB_v1", "qAB_v2 (table)", "qAB_v3", "qAB_v4"}
+        for med, p20, p80 in res.values():
+            assert 0 < p20 <= med <= p80
+    assert "kv_len" in capsys.readouterr().out
+    trace = tmp_path / "trace.json"
+    profiling.main(["--kv_len", "1024", "--k_rank", "256", "--v_rank", "512", "--profile", "--trace_path", str(trace)])
+    events = json.loads(trace.read_text())["traceEvents"]
+    names = {e.get("name", "") for e in events}
+    assert "Fused xKV with RoPE" in names and any("recon" in n or "latent" in n for n in names), "variant ranges and HIP kernels in the trace"
