@@ -453,16 +453,16 @@ def bench_c4(args, dev, vfact):
               for i in (order[0], order[B // 2], order[-1])}
     total_ms, step_q = time_loop(fn, args.steps, args.warmup)
     us = total_ms * 1e3 / args.steps
-    # the same call with the caller's splits taken as they are (no finer splitting of long splits inside the wrapper)
-    saved = gqa.REFINE_TOKENS, gqa.REFINE_TOKENS_WIDE
-    gqa.REFINE_TOKENS = gqa.REFINE_TOKENS_WIDE = 0
+    # the same call with the caller's splits taken as they are (split_cap_tokens = 0: the kernels add no splits)
+    saved = gqa.MAX_SPLIT_TOKENS, gqa.MAX_SPLIT_TOKENS_WIDE
+    gqa.MAX_SPLIT_TOKENS = gqa.MAX_SPLIT_TOKENS_WIDE = 0
     try:
         asis_ms, _ = time_loop(fn, args.steps, args.warmup)
     finally:
-        gqa.REFINE_TOKENS, gqa.REFINE_TOKENS_WIDE = saved
+        gqa.MAX_SPLIT_TOKENS, gqa.MAX_SPLIT_TOKENS_WIDE = saved
     algo_bytes = sum(lens) * per_tok
     gbs = algo_bytes / (us * 1e-6) / 1e9
-    limit = gqa.REFINE_TOKENS_WIDE if vfact else gqa.REFINE_TOKENS
+    limit = gqa.MAX_SPLIT_TOKENS_WIDE if vfact else gqa.MAX_SPLIT_TOKENS
     cpu = None
     if not args.no_cpu:
         # an eighth of every length (fp32): the scan is linear in the number of tokens, value = time x 8

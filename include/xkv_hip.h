@@ -18,6 +18,11 @@
  *   - split arithmetic (which tokens split i of a sequence covers, which splits are live) is
  *     the reference's, flash_decoding/gqa.py:95-99 and :273-281, bit for bit, with the
  *     sequence length taken from kv_lens[b] when kv_lens != NULL (ragged batch) else kv_len.
+ *   - `split_cap_tokens` (xkv_latent_stage1, xkv_merge_stage2; 0 = off): no split longer than this many tokens.  Sequence b is
+ *     then scanned with max(num_kv_splits[b], ceil(len_b / split_cap_tokens)) splits in that same arithmetic, evaluated on
+ *     the device by stage 1 and by the merge alike, so a ragged batch whose caller asks for long splits is still spread over
+ *     the whole chip.  max_splits - the split dimension of the workspaces - must then be at least ceil(kv_len /
+ *     split_cap_tokens) (XKV_EINVAL otherwise).  Split-K is exact under the merge: the result does not depend on it.
  */
 #ifndef XKV_HIP_H
 #define XKV_HIP_H
@@ -28,7 +33,7 @@
 extern "C" {
 #endif
 
-#define XKV_ABI_VERSION 3
+#define XKV_ABI_VERSION 4
 
 enum { XKV_F16 = 0, XKV_BF16 = 1, XKV_F32 = 2 };
 
@@ -125,7 +130,7 @@ int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_operand qr,
                       float* partial, float* lse,
                       void* scores_out, int scores_dtype,
                       const int32_t* num_kv_splits, const int32_t* kv_lens,
-                      int batch, int hq, int n_kv_groups, int kv_len, int max_splits,
+                      int batch, int hq, int n_kv_groups, int kv_len, int max_splits, int split_cap_tokens,
                       float sm_scale, float logit_cap, int dtype, void* stream);
 
 /* Split-K stage 1 with fused key reconstruction and RoPE:
@@ -202,7 +207,7 @@ int xkv_merge_stage2(const float* partial, const float* lse, void* out,
                      const void* vB, int64_t stride_vB_b, int64_t stride_vB_h, int64_t stride_vB_r,
                      int d_out, int vB_dtype,
                      const int32_t* num_kv_splits, const int32_t* kv_lens,
-                     int batch, int hq, int hkv, int kv_len, int max_splits, int dv,
+                     int batch, int hq, int hkv, int kv_len, int max_splits, int split_cap_tokens, int dv,
                      int64_t stride_o_b, int64_t stride_o_h, int out_dtype,
                      float* lse_out, int64_t stride_lse_b, int64_t stride_lse_h, void* stream);
 

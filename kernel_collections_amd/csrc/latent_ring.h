@@ -13,6 +13,7 @@ struct LatentParams {
   float* partial; float* lse; void* scores; int scores_dtype;
   const int32_t* num_splits; const int32_t* kv_lens;
   int hq, groups, kv_len, max_splits, total_wg;
+  int split_cap;   // > 0: no split longer than this many tokens (effective_splits)
   float sm_scale, logit_cap;
 };
 typedef LatentParams RingParams;

@@ -115,7 +115,7 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   const int b = wg / (p.groups * p.max_splits);
   const int L = p.kv_lens ? p.kv_lens[b] : p.kv_len;
   int start, end;
-  split_bounds(L, p.num_splits[b], split, start, end);
+  split_bounds(L, effective_splits(L, p.num_splits[b], p.split_cap), split, start, end);
   if (end <= start) return;
   const int hg = p.hq / p.groups, h0 = group * hg;
   const int ntiles = (end - start + TN - 1) / TN;

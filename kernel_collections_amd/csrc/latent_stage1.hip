@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void latent_stage1_kernel(const LatentParams p
 
   const int L = p.kv_lens ? p.kv_lens[b] : p.kv_len;
   int start, end;
-  split_bounds(L, p.num_splits[b], split, start, end);
+  split_bounds(L, effective_splits(L, p.num_splits[b], p.split_cap), split, start, end);
   if (end <= start) return;
 
   const int hg = p.hq / p.groups;  // heads of this kv group
@@ -357,11 +357,14 @@ static bool ptr16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) 
 extern "C" int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_operand qr, xkv_kv_operand C,
                                  xkv_kv_operand R, xkv_kv_operand V, float* partial, float* lse, void* scores_out,
                                  int scores_dtype, const int32_t* num_kv_splits, const int32_t* kv_lens, int batch,
-                                 int hq, int n_kv_groups, int kv_len, int max_splits, float sm_scale, float logit_cap,
+                                 int hq, int n_kv_groups, int kv_len, int max_splits, int split_cap_tokens, float sm_scale,
+                                 float logit_cap,
                                  int dtype, void* stream) {
   if (!qn.ptr || !C.ptr || !num_kv_splits || batch <= 0 || hq <= 0 || n_kv_groups <= 0 || kv_len <= 0 ||
       max_splits <= 0)
     return XKV_EINVAL;
+  // with a cap the longest sequence may need cdiv(kv_len, cap) splits: the workspace must have a row for each
+  if (split_cap_tokens < 0 || (split_cap_tokens > 0 && max_splits < cdiv(kv_len, split_cap_tokens))) return XKV_EINVAL;
   const bool scores_only = scores_out != nullptr;
   if (!scores_only && (!V.ptr || !partial || !lse)) return XKV_EINVAL;
   if (dtype != XKV_BF16 && dtype != XKV_F16) return XKV_EDTYPE;
@@ -391,7 +394,7 @@ extern "C" int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_oper
   p.dn = C.dim; p.dr = dr; p.dv = scores_only ? 64 : V.dim;
   p.partial = partial; p.lse = lse; p.scores = scores_out; p.scores_dtype = scores_dtype;
   p.num_splits = num_kv_splits; p.kv_lens = kv_lens;
-  p.hq = hq; p.groups = n_kv_groups; p.kv_len = kv_len; p.max_splits = max_splits;
+  p.hq = hq; p.groups = n_kv_groups; p.kv_len = kv_len; p.max_splits = max_splits; p.split_cap = split_cap_tokens;
   p.total_wg = batch * n_kv_groups * max_splits;
   p.sm_scale = sm_scale; p.logit_cap = logit_cap;
   const bool vshared = !scores_only && V.ptr == C.ptr && V.stride_b == C.stride_b && V.stride_l == C.stride_l &&

@@ -176,7 +176,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     const TB* __restrict__ vB, int64_t sVb, int64_t sVh, int64_t sVr, int d_out,
     const int32_t* __restrict__ num_kv_splits, const int32_t* __restrict__ kv_lens,
     int hq, int hkv, int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, int hpw,
-    float* __restrict__ lse_out, int64_t sLb, int64_t sLh, int d_blk) {
+    float* __restrict__ lse_out, int64_t sLb, int64_t sLh, int d_blk, int split_cap) {
   extern __shared__ float merged[];  // [G][dv], then the split weights [G][max_splits]
   __shared__ float fin[4 * 512];     // per-head-block totals of the up-projection
   // this workgroup: heads hfirst .. hfirst + G - 1 of sequence b, all of kv head kh (G = hpw divides the GQA group size)
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     d_out = d_blk;
   }
   const int L = kv_lens ? kv_lens[b] : kv_len;
-  const int ns = num_kv_splits[b];
+  const int ns = effective_splits(L, num_kv_splits[b], split_cap);
   float* wts = merged + G * dv;
   int nlive = 0;
   {
@@ -358,7 +358,7 @@ template <typename O, typename TB>
 static int launch_merge(const float* partial, const float* lse, void* out, const void* vB, int64_t sVb, int64_t sVh,
                         int64_t sVr, int d_out, const int32_t* ns, const int32_t* kl, int batch, int hq, int hkv,
                         int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, float* lse_out, int64_t sLb, int64_t sLh,
-                        hipStream_t st) {
+                        int split_cap, hipStream_t st) {
   // few splits: one workgroup per kv head (vB read once for its heads); many splits: one per query head, so that the
   // partial rows of a long sequence are spread over more CUs
   const int hpw = (max_splits > 16 || hq / hkv > 16) ? 1 : hq / hkv;
@@ -369,7 +369,7 @@ static int launch_merge(const float* partial, const float* lse, void* out, const
   if (vB && (hq / hpw) * batch < 128 && max_splits >= 64 && d_out % 32 == 0) zb = d_out >= 512 ? 4 : d_out >= 256 ? 2 : 1;
   merge_stage2_kernel<O, TB><<<dim3(hq / hpw, batch, zb), dim3(256), shm, st>>>(partial, lse, (O*)out, (const TB*)vB, sVb, sVh,
                                                                                sVr, d_out, ns, kl, hq, hkv, kv_len, max_splits,
-                                                                               dv, sOb, sOh, hpw, lse_out, sLb, sLh, d_out / zb);
+                                                                               dv, sOb, sOh, hpw, lse_out, sLb, sLh, d_out / zb, split_cap);
   return launch_status();
 }
 
@@ -476,16 +476,17 @@ extern "C" int xkv_blockdiag_q(const void* q, void* out, int batch, int hq, int 
 
 extern "C" int xkv_merge_stage2(const float* partial, const float* lse, void* out, const void* vB, int64_t sVb,
                                 int64_t sVh, int64_t sVr, int d_out, int vB_dtype, const int32_t* ns,
-                                const int32_t* kl, int batch, int hq, int hkv, int kv_len, int max_splits, int dv,
-                                int64_t sOb, int64_t sOh, int out_dtype, float* lse_out, int64_t sLb, int64_t sLh,
-                                void* stream) {
+                                const int32_t* kl, int batch, int hq, int hkv, int kv_len, int max_splits,
+                                int split_cap_tokens, int dv, int64_t sOb, int64_t sOh, int out_dtype, float* lse_out,
+                                int64_t sLb, int64_t sLh, void* stream) {
   if (!partial || !lse || !out || !ns || batch <= 0 || hq <= 0 || hkv <= 0 || max_splits <= 0 || dv <= 0)
     return XKV_EINVAL;
+  if (split_cap_tokens < 0 || (split_cap_tokens > 0 && (kv_len <= 0 || max_splits < cdiv(kv_len, split_cap_tokens)))) return XKV_EINVAL;
   if (hq % hkv || hq / hkv > 32 || dv > 512) return XKV_EUNSUPPORTED;
   if (vB && (d_out <= 0 || d_out > 512 || d_out % 8)) return XKV_EUNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
 #define XKV_MERGE(O, TB) \
-  return launch_merge<O, TB>(partial, lse, out, vB, sVb, sVh, sVr, d_out, ns, kl, batch, hq, hkv, kv_len, max_splits, dv, sOb, sOh, lse_out, sLb, sLh, st)
+  return launch_merge<O, TB>(partial, lse, out, vB, sVb, sVh, sVr, d_out, ns, kl, batch, hq, hkv, kv_len, max_splits, dv, sOb, sOh, lse_out, sLb, sLh, split_cap_tokens, st)
   const int bt = vB ? vB_dtype : XKV_BF16;
   if (bt != XKV_BF16 && bt != XKV_F16) return XKV_EDTYPE;
   switch (out_dtype) {

@@ -74,6 +74,17 @@ __host__ __device__ __forceinline__ void split_bounds(int kv_len, int num_splits
   end = e < kv_len ? e : kv_len;
 }
 
+// Split count a sequence is scanned with: the caller's, or more when `cap_tokens` > 0 and the caller's splits would be longer
+// than that (one split per cap_tokens tokens at least).  Stage 1 and the merge evaluate it from the same two device
+// integers, so they agree without any exchange; split-K is exact under the merge, so the result does not depend on it.
+__host__ __device__ __forceinline__ int effective_splits(int kv_len, int num_splits, int cap_tokens) {
+  if (cap_tokens > 0) {
+    const int need = cdiv(kv_len, cap_tokens);
+    return need > num_splits ? need : num_splits;
+  }
+  return num_splits;
+}
+
 // Reductions over the 4 lane groups {n, n+16, n+32, n+48} that share a column
 // index in the 16x16 MFMA result layout.
 __device__ __forceinline__ float group4_max(float v) {

@@ -10,37 +10,17 @@ Split ranges follow gqa.py:95-99 exactly; ``sm_scale`` multiplies the scores (gq
 """
 from __future__ import annotations
 
-import weakref
-
 import torch
 
 from kernel_collections_amd import ops
 
 
-REFINE_TOKENS = 1024        # decode_attention_fwd: longest split it runs as one workgroup (0: always the caller's splits)
-REFINE_TOKENS_WIDE = 2048   # the same for the all-heads form of decode_attention_fwd_v_factorized
-
-
-_refined = {}   # (id(splits), id(lens), tokens) -> (weakref(splits), weakref(lens), versions, result)
-
-
-def _refine_splits(splits, lens, batch, kv_len, S, tokens, device):
-    """At least one split per `tokens` tokens for every sequence: ``max(splits, ceil(len / tokens))`` on the device (no
-    host synchronisation) and the matching bound on the split count.  The result is remembered while the SAME tensor
-    objects are passed again unmodified (identity through weak references, so a freed tensor whose address is reused
-    never matches, plus the tensors' version counters), which is what a decode loop does."""
-    S2 = max(S, -(-kv_len // tokens))
-    if lens is None:
-        return torch.maximum(splits, ops.uniform_splits(batch, -(-kv_len // tokens), device)), S2
-    key = (id(splits), id(lens), tokens)
-    hit = _refined.get(key)
-    if hit is not None and hit[0]() is splits and hit[1]() is lens and hit[2] == (splits._version, lens._version):
-        return hit[3], S2
-    if len(_refined) >= 16:
-        _refined.clear()
-    out = torch.maximum(splits, ((lens + (tokens - 1)) // tokens).to(torch.int32))
-    _refined[key] = (weakref.ref(splits), weakref.ref(lens), (splits._version, lens._version), out)
-    return out, S2
+# Longest split, in tokens, that stage 1 scans as one workgroup (0: the caller's splits as they are).  The kernels raise a
+# sequence's split count to ceil(len / this) when the caller asked for fewer (`split_cap_tokens` of the C entry points):
+# split-K is exact under the merge, so the caller's count is a lower bound on the parallelism, not part of the result, and a
+# ragged batch scanned in 4096-token splits would otherwise leave most CUs idle behind its longest sequences.
+MAX_SPLIT_TOKENS = 1024
+MAX_SPLIT_TOKENS_WIDE = 2048   # the all-heads form of decode_attention_fwd_v_factorized (one workgroup serves 32 heads)
 
 
 def _prep(q, k_buffer, num_kv_splits, max_kv_splits, kv_lens):
@@ -68,16 +48,14 @@ def decode_attention_fwd(q, k_buffer, v_buffer, o, num_kv_splits, max_kv_splits,
     kv_len = k_buffer.shape[1]
     q3 = ops._q3(q)
     k_buffer, v_buffer = ops.as_rows(k_buffer), ops.as_rows(v_buffer)
-    if REFINE_TOKENS and kv_len > S * REFINE_TOKENS:
-        # shorter splits balance a ragged batch over the CUs (split-K is exact under the merge, so the caller's split
-        # count is a lower bound, not a contract on the arithmetic); computed on the device, no host synchronisation
-        splits, S = _refine_splits(splits, lens, batch, kv_len, S, REFINE_TOKENS, q.device)
+    cap = MAX_SPLIT_TOKENS
+    S = ops.capped_splits(kv_len, S, cap)     # room in the workspaces for the splits the kernels may add (host arithmetic only)
     partial, lse = ops.workspaces(batch, hq, S, dv, q.device)
     ops.latent_stage1(q3, None, None,
                       (k_buffer, k_buffer.stride(0), k_buffer.stride(1), k_buffer.stride(2), d), None,
                       (v_buffer, v_buffer.stride(0), v_buffer.stride(1), v_buffer.stride(2), dv),
-                      partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale))
-    return ops.merge_stage2(partial, lse, o, None, splits, lens, batch, hq, hq, kv_len, S)
+                      partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale), split_cap=cap)
+    return ops.merge_stage2(partial, lse, o, None, splits, lens, batch, hq, hq, kv_len, S, split_cap=cap)
 
 
 def decode_attention_fwd_v_factorized(q, k_buffer, v_A_buffer, v_B_buffer, o, num_kv_splits, max_kv_splits,
@@ -93,13 +71,10 @@ def decode_attention_fwd_v_factorized(q, k_buffer, v_A_buffer, v_B_buffer, o, nu
     k_buffer, v_A_buffer = ops.as_rows(k_buffer), ops.as_rows(v_A_buffer)
     wide = (hkv * d == 1024 and rv in (256, 384, 512)) or (hkv * d == 512 and rv == 512)
     wide = wide and hq <= 32 and k_buffer.stride(2) == d
-    if wide:
-        # One workgroup serves every head of a split, so there are hkv times fewer workgroups than in the per-head
-        # form: when the caller's splits are longer than 2048 tokens every sequence gets at least one split per 2048
-        # tokens (split-K is exact under the merge, so the caller's split count is a lower bound, not a contract on
-        # the arithmetic).  Computed on the device: no host synchronisation.
-        if REFINE_TOKENS_WIDE and kv_len > S * REFINE_TOKENS_WIDE:
-            splits, S = _refine_splits(splits, lens, batch, kv_len, S, REFINE_TOKENS_WIDE, q.device)
+    # one workgroup serves every head of a split in the wide form, so there are hkv times fewer workgroups than in the
+    # per-head form: its splits may be twice as long before the chip runs out of work
+    cap = MAX_SPLIT_TOKENS_WIDE if wide else 0
+    S = ops.capped_splits(kv_len, S, cap)
     partial, lse = ops.workspaces(batch, hq, S, rv, q.device)
     if wide:
         # all heads from one workgroup: the token's keys are one hkv*d-wide row against a block-diagonal query, and the
@@ -108,10 +83,10 @@ def decode_attention_fwd_v_factorized(q, k_buffer, v_A_buffer, v_B_buffer, o, nu
         ops.latent_stage1(qbd, None, None,
                           (k_buffer, k_buffer.stride(0), k_buffer.stride(1), 0, hkv * d), None,
                           (v_A_buffer, v_A_buffer.stride(0), v_A_buffer.stride(1), 0, rv),
-                          partial, lse, None, splits, lens, batch, hq, 1, kv_len, S, float(sm_scale))
+                          partial, lse, None, splits, lens, batch, hq, 1, kv_len, S, float(sm_scale), split_cap=cap)
     else:
         ops.latent_stage1(q3, None, None,
                           (k_buffer, k_buffer.stride(0), k_buffer.stride(1), k_buffer.stride(2), d), None,
                           (v_A_buffer, v_A_buffer.stride(0), v_A_buffer.stride(1), 0, rv),
                           partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale))
-    return ops.merge_stage2(partial, lse, o, v_B_buffer, splits, lens, batch, hq, hkv, kv_len, S)
+    return ops.merge_stage2(partial, lse, o, v_B_buffer, splits, lens, batch, hq, hkv, kv_len, S, split_cap=cap)

@@ -174,14 +174,16 @@ def blockdiag_q(q3: torch.Tensor, hkv: int) -> torch.Tensor:
 
 
 def latent_stage1(qn, qn_lo, qr, C, R, V, partial, lse, scores, num_kv_splits, kv_lens,
-                  batch, hq, groups, kv_len, max_splits, sm_scale, logit_cap=0.0):
-    """C / R / V are `(tensor, stride_b, stride_l, stride_h, dim)` tuples or None."""
+                  batch, hq, groups, kv_len, max_splits, sm_scale, logit_cap=0.0, split_cap=0):
+    """C / R / V are `(tensor, stride_b, stride_l, stride_h, dim)` tuples or None.  `split_cap` > 0: no split longer than that
+    many tokens (the kernels then scan sequence b with ``max(num_kv_splits[b], ceil(len_b / split_cap))`` splits; `max_splits`,
+    the split dimension of the workspaces, must cover ``ceil(kv_len / split_cap)``)."""
     def op(x):
         return kv_operand(None) if x is None else kv_operand(*x)
     sd = dtype_code(scores.dtype) if scores is not None else 0
     check(_lib.lib().xkv_latent_stage1(
         q_operand(qn), ptr(qn_lo), q_operand(qr), op(C), op(R), op(V), ptr(partial), ptr(lse), ptr(scores), sd,
-        ptr(num_kv_splits), ptr(kv_lens), batch, hq, groups, kv_len, max_splits,
+        ptr(num_kv_splits), ptr(kv_lens), batch, hq, groups, kv_len, max_splits, int(split_cap),
         c_float(sm_scale), c_float(logit_cap), dtype_code(qn.dtype), stream_ptr(qn)), "xkv_latent_stage1")
 
 
@@ -204,7 +206,7 @@ def recon_stage1(q3, kA, kB, vA, partial, lse, scores, num_kv_splits, kv_lens, b
         "xkv_recon_stage1")
 
 
-def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, kv_len, max_splits, lse_out=None):
+def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, kv_len, max_splits, lse_out=None, split_cap=0):
     """out `[b,Hq,*]` (strides honoured on the first two axes).  `lse_out` `[b,Hq]` (any strides, fp32): log-sum-exp
     of the merged range.  Up-projections wider than 512 columns run as column blocks of 512."""
     dv = partial.shape[-1]
@@ -214,7 +216,7 @@ def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, 
     def call(o, w, d_out, sv, vdt, lo):
         check(_lib.lib().xkv_merge_stage2(
             ptr(partial), ptr(lse), ptr(o), ptr(w), c_int64(sv[0]), c_int64(sv[1]), c_int64(sv[2]), d_out, vdt,
-            ptr(num_kv_splits), ptr(kv_lens), batch, hq, hkv, kv_len, max_splits, dv,
+            ptr(num_kv_splits), ptr(kv_lens), batch, hq, hkv, kv_len, max_splits, int(split_cap), dv,
             c_int64(o.stride(0)), c_int64(o.stride(1)), dtype_code(o.dtype), ptr(lo), c_int64(sl[0]), c_int64(sl[1]),
             stream_ptr(partial)), "xkv_merge_stage2")
 
@@ -227,6 +229,11 @@ def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, 
         c1 = min(c0 + 512, vB.shape[-1])
         call(out[..., c0:c1], vB[..., c0:c1], c1 - c0, sv, vdt, lse_out if c0 == 0 else None)
     return out
+
+
+def capped_splits(kv_len: int, max_kv_splits: int, cap_tokens: int) -> int:
+    """Split dimension of the workspaces when no split may be longer than `cap_tokens` tokens (0: no cap)."""
+    return max(int(max_kv_splits), _cdiv(kv_len, cap_tokens)) if cap_tokens else int(max_kv_splits)
 
 
 def workspaces(batch: int, hq: int, max_splits: int, dv: int, device):

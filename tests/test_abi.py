@@ -42,7 +42,7 @@ def test_argument_errors_are_reported_before_any_launch():
     ns = ctypes.c_void_p(16)
     # feature width 100 is outside the envelope (multiple of 32 required)
     rc = L.xkv_latent_stage1(q, null, _lib.QOperand(null, 0), kv, none, kv, ctypes.c_void_p(16), ctypes.c_void_p(16),
-                             null, 0, ns, null, 1, 4, 1, 8, 1, 1.0, 0.0, _lib.XKV_BF16, null)
+                             null, 0, ns, null, 1, 4, 1, 8, 1, 0, 1.0, 0.0, _lib.XKV_BF16, null)
     assert rc == -2
     with pytest.raises(RuntimeError, match="envelope"):
         _lib.check(rc, "xkv_latent_stage1")
@@ -138,27 +138,23 @@ def test_settled_splits_leaves_no_dead_split():
             assert len(live) == s and live[0][1] == 0 and live[-1][2] == L, (L, n, s)
 
 
-def test_refined_splits_follow_the_lengths_and_their_updates():
-    """The plain and V-factorised decode wrappers give every sequence at least one split per N tokens; the device-side
-    result is remembered only while the caller's tensors are unmodified."""
-    from kernel_collections_amd.flash_decoding import gqa
-    lens = torch.tensor([1, 1024, 1025, 5000, 104212], dtype=torch.int32)
-    splits = torch.tensor([1, 1, 1, 2, 26], dtype=torch.int32)
-    out, S = gqa._refine_splits(splits, lens, 5, 104212, 26, 1024, lens.device)
-    assert out.dtype == torch.int32 and out.tolist() == [1, 1, 2, 5, 102] and S == 102
-    again, _ = gqa._refine_splits(splits, lens, 5, 104212, 26, 1024, lens.device)
-    assert again is out                                   # same tensors, same versions: no new device work
-    lens[3] = 9000                                        # an in-place update must not see the remembered result
-    out2, _ = gqa._refine_splits(splits, lens, 5, 104212, 26, 1024, lens.device)
-    assert out2.tolist() == [1, 1, 2, 9, 102]
-    splits[0] = 7                                         # the caller's own count is a lower bound
-    out3, S3 = gqa._refine_splits(splits, lens, 5, 104212, 200, 1024, lens.device)
-    assert out3.tolist() == [7, 1, 2, 9, 102] and S3 == 200
-    other = torch.tensor([4000, 10, 10, 10, 10], dtype=torch.int32)    # another tensor object never sees a remembered result
-    out4, _ = gqa._refine_splits(splits, other, 5, 104212, 26, 1024, lens.device)
-    assert out4.tolist() == [7, 1, 1, 2, 26]
-    uni, Su = gqa._refine_splits(torch.full((3,), 2, dtype=torch.int32), None, 3, 5000, 2, 2048, lens.device)
-    assert uni.tolist() == [3, 3, 3] and Su == 3
+def test_split_cap_needs_room_in_the_workspace():
+    """With split_cap_tokens > 0 a sequence may be scanned with ceil(kv_len / cap) splits: stage 1 and the merge refuse
+    (before any launch) a workspace whose split dimension is smaller, and accept one that covers it."""
+    from kernel_collections_amd import _lib, ops
+    L = _lib.lib()
+    null, p16 = ctypes.c_void_p(0), ctypes.c_void_p(16)
+    q = _lib.QOperand(p16, 128)
+    kv = _lib.KVOperand(p16, 8192 * 128, 128, 0, 128)
+    none = _lib.KVOperand(null, 0, 0, 0, 0)
+    args = lambda max_splits, cap: (q, null, _lib.QOperand(null, 0), kv, none, kv, p16, p16, null, 0, p16, null,
+                                    1, 4, 1, 8192, max_splits, cap, 1.0, 0.0, _lib.XKV_BF16, null)
+    assert L.xkv_latent_stage1(*args(7, 1024)) == -1          # 8192 tokens at 1024 per split need 8 rows
+    assert L.xkv_latent_stage1(*args(2, -5)) == -1
+    assert L.xkv_merge_stage2(p16, p16, p16, null, 0, 0, 0, 128, 0, p16, null, 1, 4, 1, 8192, 7, 1024, 128, 512, 128, _lib.XKV_BF16,
+                              null, 0, 0, null) == -1
+    assert ops.capped_splits(8192, 2, 1024) == 8 and ops.capped_splits(8192, 16, 1024) == 16 and ops.capped_splits(8192, 2, 0) == 2
+    assert ops.capped_splits(104212, 26, 1024) == 102
 
 
 REFERENCE_IMPORTS = """

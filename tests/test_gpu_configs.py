@@ -69,8 +69,8 @@ def test_ragged_4096_token_splits_with_long_sequences(dev, dtype, monkeypatch):
     outs = {}
     for tokens in ("default", 0):
         if tokens == 0:
-            monkeypatch.setattr(gqa, "REFINE_TOKENS", 0)
-            monkeypatch.setattr(gqa, "REFINE_TOKENS_WIDE", 0)
+            monkeypatch.setattr(gqa, "MAX_SPLIT_TOKENS", 0)
+            monkeypatch.setattr(gqa, "MAX_SPLIT_TOKENS_WIDE", 0)
         o = torch.zeros_like(q)
         gqa.decode_attention_fwd(q, K, V, o, nst, S, scale, kv_lens=kl)
         check_out(o, ref, f"ragged plain, long splits ({tokens})")
