@@ -216,8 +216,10 @@ int xkv_merge_stage2(const float* partial, const float* lse, void* out,
  * xkv_ceiling_mfma: every wave of `workgroups` x 256 threads issues iters x 32 v_mfma_f32_32x32x16 (dtype XKV_BF16 / XKV_F16) on
  *   register operands, four independent accumulator chains; FLOP = workgroups * 4 * iters * 32 * 32768.  out: workgroups * 256 floats.
  * xkv_ceiling_stream: reads the first workgroups * 4 * 8192 * floor(bytes / (workgroups * 4 * 8192)) bytes of src once, each wave
- *   its own contiguous share in 8 KiB steps, into registers (to_lds == 0) or straight into a per-wave LDS ring of `depth` steps
- *   (2, 3 or 4; depth - 1 steps in flight) that nothing reads.  out: 256 floats. */
+ *   its own contiguous share in 8 KiB steps, into registers (to_lds == 0), straight into a per-wave LDS ring of `depth` steps
+ *   (to_lds == 1; depth 2, 3 or 4; depth - 1 steps in flight) that nothing reads, or into a register queue `depth` steps deep (to_lds
+ *   == 2; depth 2, 4 or 6) whose steps are written on to LDS with ds_write_b128 as they land.  out: 256 floats
+ *   (to_lds == 2: workgroups * 256 floats, the number of 16-byte packets each thread handed on). */
 int xkv_ceiling_mfma(float* out, int workgroups, int iters, int dtype, void* stream);
 int xkv_ceiling_stream(const void* src, int64_t bytes, int workgroups, int to_lds, int depth, float* out, void* stream);
 

@@ -79,6 +79,44 @@ __global__ __launch_bounds__(256) void ceiling_stream_kernel(const unsigned char
   if (fold == 0x12345678u || blockIdx.x == 0) out[threadIdx.x] = (float)fold;
 }
 
+// The third path: 16-byte loads into a register queue DEPTH steps deep (so DEPTH x 8 KiB per wave are in flight whatever the
+// LDS holds), each step written on to a small per-wave LDS buffer with ds_write_b128 once it has landed - what a loader wave
+// does when registers, not LDS slots, are the landing zone.
+template <int DEPTH>
+__global__ __launch_bounds__(256) void ceiling_stream_regs_to_lds_kernel(const unsigned char* __restrict__ src, int64_t steps_per_wave,
+                                                                         float* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t wave_id = (int64_t)blockIdx.x * 4 + wave;
+  const u32x4* base = reinterpret_cast<const u32x4*>(src + wave_id * steps_per_wave * 8192) + lane;
+  u32x4* buf = reinterpret_cast<u32x4*>(smem + wave * 2 * 8192) + lane;   // two 8 KiB buffers per wave
+  u32x4 v[DEPTH][8];
+  unsigned seen = 0;   // 16-byte packets handed on (their first and last words agree in a buffer filled with one byte value)
+  const int64_t rounds = steps_per_wave / DEPTH;
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+    for (int r = 0; r < 8; ++r) v[d][r] = __builtin_nontemporal_load(base + (int64_t)d * 512 + r * 64);
+  for (int64_t k = 0; k < rounds; ++k) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      u32x4* dst = buf + (d & 1) * 512;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        dst[r * 64] = v[d][r];     // the oldest step has landed: hand it on
+        seen += v[d][r][0] == v[d][r][3] ? 1u : 0u;
+      }
+      if (k + 1 < rounds) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) v[d][r] = __builtin_nontemporal_load(base + ((k + 1) * DEPTH + d) * 512 + r * 64);
+      }
+    }
+  }
+  __syncthreads();
+  out[(size_t)blockIdx.x * 256 + threadIdx.x] = (float)seen;   // host check: the sum is bytes / 16
+}
+
 template <bool TO_LDS, int DEPTH>
 static int launch_stream(const void* src, int64_t bytes, int wgs, float* out, hipStream_t st) {
   const int64_t steps = bytes / ((int64_t)wgs * 4 * 8192);
@@ -112,6 +150,18 @@ extern "C" int xkv_ceiling_stream(const void* src, int64_t bytes, int workgroups
   if (reinterpret_cast<uintptr_t>(src) & 15) return XKV_EALIGN;
   hipStream_t st = (hipStream_t)stream;
   if (!to_lds) return launch_stream<false, 1>(src, bytes, workgroups, out, st);
+  if (to_lds == 2) {   // register queue of `depth` steps, then ds_write
+    const int64_t steps = bytes / ((int64_t)workgroups * 4 * 8192) / (depth > 0 ? depth : 1) * (depth > 0 ? depth : 1);
+    if (steps <= 0) return XKV_EINVAL;
+    const unsigned char* s8 = reinterpret_cast<const unsigned char*>(src);
+    switch (depth) {
+      case 2: ceiling_stream_regs_to_lds_kernel<2><<<dim3(workgroups), dim3(256), 4 * 2 * 8192, st>>>(s8, steps, out); break;
+      case 4: ceiling_stream_regs_to_lds_kernel<4><<<dim3(workgroups), dim3(256), 4 * 2 * 8192, st>>>(s8, steps, out); break;
+      case 6: ceiling_stream_regs_to_lds_kernel<6><<<dim3(workgroups), dim3(256), 4 * 2 * 8192, st>>>(s8, steps, out); break;
+      default: return XKV_EUNSUPPORTED;
+    }
+    return launch_status();
+  }
   switch (depth) {
     case 2: return launch_stream<true, 2>(src, bytes, workgroups, out, st);
     case 3: return launch_stream<true, 3>(src, bytes, workgroups, out, st);
