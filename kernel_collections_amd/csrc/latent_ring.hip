@@ -3,21 +3,22 @@
 // factorised decode with the per-head keys viewed as one 1024-wide row against a block-diagonal query).
 //
 // Same arithmetic as latent_stage1.hip; what differs is how bytes move.  A CU has to keep roughly
-// (HBM latency x its share of the HBM rate) = 60-100 KB of loads in flight to stream at full rate, which a
-// register-staged double buffer cannot hold.  Here the token rows go HBM -> LDS directly
-// (global_load_lds_dwordx4, no VGPRs involved) into a ring of RSLOT tiles of TN tokens, RSLOT-1 tiles always in
-// flight, one workgroup per CU, and the query operands live in registers for the whole kernel.  The loads are issued by
-// two extra wavefronts that do nothing else (a load instruction that stalls on a full memory queue then never holds up
-// the arithmetic); they take part in the same barriers.  Per tile:
-//   A:  loaders wait for tile t; barrier; loaders issue tile t+RSLOT-1 into the slot PV(t-1) just released
+// (HBM latency x its share of the HBM rate) = 60-100 KB of loads in flight to stream at full rate.  Here four extra
+// wavefronts do nothing but move token rows: plain 16-byte vector loads into a register queue of RING_QD tiles per wave
+// (that queue is what is in flight), then ds_write_b128 into a two-slot ring of TN-token tiles in the LDS.  A load
+// instruction that stalls on a full memory queue then never holds up the arithmetic; the loader waves take part in the
+// same barriers.  One workgroup per CU; the query operands live in registers for the whole kernel.  Per tile t:
+//   A:  barrier (slot of tile t-1 is free); loaders wait for tile t+1 only, write it into that slot, refill the queue entry
 //   QK: wave (tb, kh) multiplies token block tb by its k-range kh of q on v_mfma_f32_16x16x32 -> partial scores in LDS
 //   B:  barrier; softmax threads add the k-range partials, update the running max / sum, publish P and alpha
 //   C:  barrier; PV: each wave owns a quarter of the value features, token-major operand via ds_read_b64_tr_b16.
 // Scores-only mode (qAB without PE) stops after B and writes the summed scores.
+// The start of the kernel is latency, not bandwidth: the loader branch comes first in the code and addresses its rows
+// with scalar arithmetic so that the first loads leave as early as possible.
 //
 // LDS tile layout: C (and V) rows are row-major with a 16-byte pad (conflict-free ds_read_b128 over 16 rows and
-// conflict-free transposed reads); the 128-byte RoPE-key rows are stored chunk-major ([8 chunks][TN rows][16 B]),
-// which the per-lane global addresses of the direct-to-LDS load make free.
+// conflict-free transposed reads); the 128-byte RoPE-key rows are stored chunk-major ([8 chunks][TN rows][16 B]):
+// lane l of loader wave w fetches chunk 2w + l/32 of row l%32 and writes it at l * 16 of that wave's 1 KiB piece.
 #include "xkv_common.h"
 #include "latent_ring.h"
 
@@ -27,11 +28,22 @@ typedef short s16x4r __attribute__((ext_vector_type(4)));
 typedef short s16x8r __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4r __attribute__((ext_vector_type(4)));
 
-// LDS destination of a direct-to-LDS load = M0 + lane * 16; a SALU write of M0 needs one wait state before its use.
-__device__ __forceinline__ void ring_load16(const void* sbase, unsigned voff, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase)
-               : "memory", "m0");
+// Streaming 16-byte load the compiler does not track: the register queue of the loader waves is drained with explicit
+// vmcnt waits (the compiler's own counting gives up at the loop back edge and would drain the whole queue per tile).
+// The value must pass through ring_landed() after the wait and before its first use.  A wave that uses these must not
+// issue any other vector-memory load.
+__device__ __forceinline__ u32x4 ring_ldg(const void* p) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(v) : "v"(p));
+  return v;
 }
+// the same with a wave-uniform base in SGPRs and a 32-bit per-lane offset: the row addresses then cost SALU work only
+template <int OFF> __device__ __forceinline__ u32x4 ring_ldg_s(const void* sbase, unsigned voff) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3 nt" : "=v"(v) : "v"(voff), "s"(sbase), "n"(OFF));
+  return v;
+}
+__device__ __forceinline__ void ring_landed(u32x4& v) { asm volatile("" : "+v"(v)); }
 template <int N> __device__ __forceinline__ void ring_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
 __device__ __forceinline__ s16x4r ring_tr4(const unsigned char* p) {
@@ -46,6 +58,13 @@ __device__ __forceinline__ f32x4 mfma16k16(_Float16, s16x4r a, s16x4r b, f32x4 c
   return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4r, a), __builtin_bit_cast(f16x4r, b), c, 0, 0, 0);
 }
 
+#ifdef XKV_RING_STAMPS
+__device__ unsigned long long ring_stamps[4096 * 8];
+#define STAMP(i) do { if (lane == 0) ring_stamps[(blockIdx.x & 4095) * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define STAMP(i)
+#endif
+constexpr int RING_QD = 2;      // tiles per loader wave in flight in registers (deeper queues only lengthen the start)
 enum { RING_SCORES = 0, RING_VSHARED = 1, RING_VDISTINCT = 2, RING_VHEADS = 3 };
 constexpr int RING_DVH = 128;   // head width of the per-head value rows (RING_VHEADS)
 
@@ -62,7 +81,7 @@ struct RingShape {
   static constexpr int SP = TN + 4;                        // partial-score row stride (floats)
   static constexpr int LDP = TN + 8;                       // P row stride (elements)
   static constexpr int TAIL = KSPLIT * HB * SP * 4 + HB * LDP * 2 + HB * 4 + HB * 8;
-  static constexpr int RSLOT = (4 * SLOT + TAIL <= 160 * 1024) ? 4 : 3;
+  static constexpr int RSLOT = 2;                          // the tile being read and the tile being written
   static constexpr int SHM = RSLOT * SLOT + TAIL;
   static_assert(SHM <= 160 * 1024, "ring does not fit the LDS");
 };
@@ -72,8 +91,8 @@ struct RingShape {
 // DN features of the C row / V is a second, DVW-wide row stream / V is a second stream of DVW / 128 per-kv-head value
 // rows of 128 features (plain values under absorbed factorised keys): the workgroup serves every query head, wave w
 // accumulates kv heads 2w, 2w+1, and query head h multiplies the values of kv head h / (heads per kv head).
-template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE, int DVW, int NLOAD>
-__global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const RingParams p) {
+template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE, int DVW>
+__global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
   typedef typename Elem<T>::vec8 vec8;
   typedef RingShape<TN, DN, HAS_R, VMODE, NHB, DVW> S;
   constexpr bool SCORES = VMODE == RING_SCORES, V2 = VMODE >= RING_VDISTINCT, VHEADS = VMODE == RING_VHEADS;
@@ -85,15 +104,14 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   constexpr int KS_W = NKS / KSPLIT;              // k-steps per wave
   static_assert(NKS % KSPLIT == 0, "the k-ranges are equal");
   static_assert(!HAS_R || TN == 32, "RoPE-key rows need 32-token tiles");
+  static_assert(DN <= 1024 && DVW <= 1024, "a row takes at most two load instructions");
   constexpr int IPR = DN > 512 ? DN / 512 : 1;    // load instructions per C row (1 KiB each; rows under 1 KiB use DN/8 lanes)
   constexpr bool CPART = DN < 512;               // a C row fills only part of a load instruction
-  // who issues the tile loads: the four compute waves (NLOAD == 0) or NLOAD extra waves that do nothing else, so that a
-  // load instruction stalled on a full memory queue never holds up the MFMA / softmax work
-  constexpr int NISS = NLOAD ? NLOAD : 4;
-  constexpr int RPW = TN / NISS;                  // rows per issuing wave per tile
-  constexpr int RIW = 4 / NISS;                   // RoPE-key load instructions per issuing wave (4 per tile)
-  constexpr int LPT = RPW * IPR + (HAS_R ? RIW : 0) + (V2 ? RPW * VIPR : 0);   // loads per issuing wave per tile
-  constexpr int WAITN = (RSLOT - 2) * LPT < 63 ? (RSLOT - 2) * LPT : 63;   // vmcnt holds 6 bits
+  // waves 4..7 move the tile rows; each brings TN/4 rows of C (and V) and two 16-byte chunks of every RoPE-key row
+  constexpr int QD = RING_QD;
+  constexpr int RPW = TN / 4;                     // rows per loader wave per tile
+  constexpr int LPT = RPW * IPR + (HAS_R ? 1 : 0) + (V2 ? RPW * VIPR : 0);   // loads per loader wave per tile
+  static_assert((QD - 1) * LPT <= 63, "vmcnt holds 6 bits");
   constexpr int DV = VMODE == RING_VSHARED ? DN : VHEADS ? RING_DVH : DVW;   // value features of an output row
   constexpr int NVB = VHEADS ? RING_DVH / 16 : DV / 64;   // 16-feature blocks per wave (per kv head under VHEADS)
   constexpr int NA2 = VHEADS ? KVW : NHB;
@@ -106,8 +124,9 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n16 = lane & 15, g4 = lane >> 4;
   const int tb = wave % NTB, kh = wave / NTB;
-  const int iw = NLOAD ? wave - 4 : wave;         // index among the issuing waves (negative: not an issuer)
+  const int iw = wave - 4;                        // index among the loader waves (negative: a compute wave)
 
+  if (wave == 0) STAMP(0);
   const int wg = xcd_cluster_remap(blockIdx.x, p.groups);   // the kv groups of one (sequence, split) share an L2
   if (wg >= p.total_wg) return;
   const int group = wg % p.groups;
@@ -120,6 +139,7 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   const int hg = p.hq / p.groups, h0 = group * hg;
   const int ntiles = (end - start + TN - 1) / TN;
   const int last = end - 1;
+  if (wave == 0) STAMP(1);
 
   // ---- LDS carve-up -------------------------------------------------------------------------------------------
   unsigned char* ring = smem;
@@ -127,7 +147,6 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   T* p_lds = reinterpret_cast<T*>(s_part + KSPLIT * HB * SP);      // [HB][LDP]
   float* alpha_lds = reinterpret_cast<float*>(p_lds + HB * LDP);   // [HB]
   float* ml_lds = alpha_lds + HB;                                  // [HB][2]
-  const unsigned ring_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)ring;
 
   // ---- tile loads: wave w brings rows RPW w .. +RPW of C (and V) and RoPE-key chunks 2w, 2w+1 of every row ---------
   const unsigned char* Cb = reinterpret_cast<const unsigned char*>(p.C) + (b * p.sCb + group * p.sCh) * 2;
@@ -137,71 +156,78 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   const int64_t crow_bytes = p.sCl * 2, rrow_bytes = p.sRl * 2, vrow_bytes = p.sVl * 2;
   const unsigned lane_off = lane * 16;
   const int r_row = lane & 31;
-  auto issue_tile = [&](int t) {
-    const unsigned slot = ring_lds + (unsigned)(t % RSLOT) * SLOT;
-    const int base = start + t * TN;
-    const int tok0 = base + iw * RPW;
-    if (base + TN <= end) {            // whole tile inside the split: row pointers advance by adds
-      const unsigned char* row = Cb + (int64_t)tok0 * crow_bytes;
+  if (__builtin_expect(wave >= 4, 1)) {   // laid out first: the sooner the first loads are issued, the shorter the start
+    u32x4 rq[QD][LPT];
+    auto fetch = [&](int t, u32x4 (&q)[LPT]) {
+      const int base = start + t * TN;
+      int n = 0;
 #pragma unroll
       for (int r = 0; r < RPW; ++r) {
-#pragma unroll
-        for (int c = 0; c < IPR; ++c)
-          if (!CPART || lane < DN / 8) ring_load16(row + c * 1024, lane_off, slot + (iw * RPW + r) * CROW + c * 1024);
-        row += crow_bytes;
-      }
-      if (V2) {
-        const unsigned char* vrow = Vb + (int64_t)tok0 * vrow_bytes;
-#pragma unroll
-        for (int r = 0; r < RPW; ++r) {
-#pragma unroll
-          for (int c = 0; c < VIPR; ++c)
-            if (DVW >= 512 || lane < DVW / 8)
-              ring_load16(vrow + c * 1024, lane_off, slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW + c * 1024);
-          vrow += vrow_bytes;
+        int tok = base + iw * RPW + r;
+        tok = tok < last ? tok : last;   // rows past the split end are masked in the softmax; keep the read in bounds
+        const unsigned char* row = Cb + (int64_t)tok * crow_bytes;   // wave-uniform
+        if (!CPART || lane < DN / 8) {
+          q[n] = ring_ldg_s<0>(row, lane_off);
+          if (IPR > 1) q[n + 1] = ring_ldg_s<1024>(row, lane_off);
+        }
+        n += IPR;
+        if (V2) {
+          const unsigned char* vrow = Vb + (int64_t)tok * vrow_bytes;
+          if (DVW >= 512 || lane < DVW / 8) {
+            q[n] = ring_ldg_s<0>(vrow, lane_off);
+            if (VIPR > 1) q[n + 1] = ring_ldg_s<1024>(vrow, lane_off);
+          }
+          n += VIPR;
         }
       }
-    } else {
+      if (HAS_R) {                       // this wave brings chunks 2 iw, 2 iw + 1 of every row
+        int tok = base + r_row;
+        tok = tok < last ? tok : last;
+        q[n] = ring_ldg(Rb + (int64_t)tok * rrow_bytes + (2 * iw + (lane >> 5)) * 16);
+      }
+    };
+    auto hand_on = [&](int t, u32x4 (&q)[LPT]) {   // the oldest tile of the queue: QD-1 younger ones stay in flight
+      unsigned char* slot = ring + (t % RSLOT) * SLOT + lane_off;
+      ring_wait<(QD - 1) * LPT>();
+#pragma unroll
+      for (int i = 0; i < LPT; ++i) ring_landed(q[i]);
+      int n = 0;
 #pragma unroll
       for (int r = 0; r < RPW; ++r) {
-        int tok = tok0 + r;
-        tok = tok < last ? tok : last;   // rows past the split end are masked in the softmax; keep the read in bounds
-        const unsigned char* row = Cb + (int64_t)tok * crow_bytes;
 #pragma unroll
-        for (int c = 0; c < IPR; ++c)
-          if (!CPART || lane < DN / 8) ring_load16(row + c * 1024, lane_off, slot + (iw * RPW + r) * CROW + c * 1024);
+        for (int c = 0; c < IPR; ++c, ++n)
+          if (!CPART || lane < DN / 8) st16(slot + (iw * RPW + r) * CROW + c * 1024, q[n]);
         if (V2) {
 #pragma unroll
-          for (int c = 0; c < VIPR; ++c)
-            if (DVW >= 512 || lane < DVW / 8)
-              ring_load16(Vb + (int64_t)tok * vrow_bytes + c * 1024, lane_off,
-                          slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW + c * 1024);
+          for (int c = 0; c < VIPR; ++c, ++n)
+            if (DVW >= 512 || lane < DVW / 8) st16(slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW + c * 1024, q[n]);
+        }
+      }
+      if (HAS_R) st16(slot + CBYTES + iw * 1024, q[n]);
+    };
+    if (wave == 4) STAMP(2);
+#pragma unroll
+    for (int d = 0; d < QD; ++d) {
+      fetch(d, rq[d]);
+      if (wave == 4 && d == 0) STAMP(5);
+    }
+    if (wave == 4) STAMP(7);
+    hand_on(0, rq[0]);                               // the ring starts empty
+    fetch(QD, rq[0]);
+    // During tile t the loader hands tile t+1 on (its slot was released by barrier A) and refills that queue entry: the
+    // look-ahead lives in the queue, a tile is waited for only when the next iteration needs it.
+    for (int t = 0; t < ntiles; t += QD) {          // t stays a multiple of QD, so every queue index below is static
+#pragma unroll
+      for (int u = 0; u < QD; ++u) {
+        if (t + u < ntiles) {
+          __syncthreads();                           // A: the slot of tile t+u-1 is free
+          hand_on(t + u + 1, rq[(u + 1) % QD]);
+          fetch(t + u + 1 + QD, rq[(u + 1) % QD]);
+          __syncthreads();                           // B
+          if (!SCORES) __syncthreads();              // C
         }
       }
     }
-    if (HAS_R) {
-      int tok = base + r_row;
-      tok = tok < last ? tok : last;
-#pragma unroll
-      for (int j = 0; j < RIW; ++j) {   // instruction w of 4 brings chunks 2w, 2w+1 of every row
-        const int w = iw * RIW + j;
-        ring_load16(Rb, (unsigned)tok * (unsigned)rrow_bytes + (2 * w + (lane >> 5)) * 16, slot + CBYTES + w * 1024);
-      }
-    }
-  };
-  if (iw >= 0) {
-#pragma unroll
-    for (int t = 0; t < RSLOT - 1; ++t) issue_tile(t);
-  }
-  if (NLOAD && wave >= 4) {            // loader wave: keep RSLOT-1 tiles in flight, take part in every barrier of the loop
-    for (int t = 0; t < ntiles; ++t) {
-      ring_wait<WAITN>();              // tile t has landed
-      __syncthreads();                 // A
-      issue_tile(t + RSLOT - 1);
-      __syncthreads();                 // B
-      if (!SCORES) __syncthreads();    // C
-    }
-    ring_wait<0>();
     return;
   }
 
@@ -209,28 +235,24 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   vec8 qreg[KS_W][NHB], qlo[LO ? KS_W : 1][NHB];
   const int ks0 = kh * KS_W;
 #pragma unroll
-  for (int k = 0; k < KS_W; ++k) {
-    const int ks = ks0 + k;
+  for (int hb = 0; hb < NHB; ++hb) {
+    int row = hb * 16 + n16;
+    row = row < hg ? row : hg - 1;   // head rows past the group repeat its last row: finite values that are never written out
+    const int64_t qh = (int64_t)b * p.hq + h0 + row;
+    const T* qn_l = reinterpret_cast<const T*>(p.qn) + qh * DN + ks0 * 32 + 8 * g4;
+    const T* ql_l = LO ? reinterpret_cast<const T*>(p.qn_lo) + qh * DN + ks0 * 32 + 8 * g4 : nullptr;
+    const T* qr_l = HAS_R ? reinterpret_cast<const T*>(p.qr) + qh * 64 + (ks0 - NKS_N) * 32 + 8 * g4 : nullptr;
 #pragma unroll
-    for (int hb = 0; hb < NHB; ++hb) {
-      const int row = hb * 16 + n16;
-      vec8 v = {0, 0, 0, 0, 0, 0, 0, 0}, vl = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (row < hg) {
-        const int64_t qh = (int64_t)b * p.hq + h0 + row;
-        if (ks < NKS_N) {
-          v = ld16<vec8>(reinterpret_cast<const T*>(p.qn) + qh * DN + ks * 32 + 8 * g4);
-          if (LO) vl = ld16<vec8>(reinterpret_cast<const T*>(p.qn_lo) + qh * DN + ks * 32 + 8 * g4);
-        } else {
-          v = ld16<vec8>(reinterpret_cast<const T*>(p.qr) + qh * 64 + (ks - NKS_N) * 32 + 8 * g4);
-        }
+    for (int k = 0; k < KS_W; ++k) {
+      if (!HAS_R || ks0 + k < NKS_N) {
+        qreg[k][hb] = ld16<vec8>(qn_l + k * 32);
+        if (LO) qlo[k][hb] = ld16<vec8>(ql_l + k * 32);
+      } else {
+        qreg[k][hb] = ld16<vec8>(qr_l + k * 32);
       }
-      qreg[k][hb] = v;
-      if (LO) qlo[k][hb] = vl;
     }
   }
-  // The compiler cannot see the direct-to-LDS loads, so any vmcnt wait it places drains them too.  Make it wait for the
-  // query loads here, once, instead of before their first use inside the loop (where it would stall every tile on
-  // the tile in flight).
+  // Wait for the query loads here, once, rather than at their first uses inside the loop.
 #pragma unroll
   for (int k = 0; k < KS_W; ++k)
 #pragma unroll
@@ -239,6 +261,7 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
       if (LO) asm volatile("" : "+v"(qlo[k][hb]));
     }
 
+  if (wave == 0) STAMP(3);
   // ---- running state ---------------------------------------------------------------------------------------------
   const int srow = tid / TPH, ssub = tid % TPH;
   float m_run = NEG_INF, l_run = 0.f;
@@ -251,9 +274,8 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   const int vcol0 = wave * (DV / 4);
 
   for (int t = 0; t < ntiles; ++t) {
-    if (!NLOAD) ring_wait<WAITN>();   // this wave's rows of tile t have landed (RSLOT-2 younger tiles may be in flight)
-    __syncthreads();                  // A: tile t complete for every wave; every wave is past PV / score write of tile t-1
-    if (!NLOAD) issue_tile(t + RSLOT - 1);   // into the slot of tile t-1 (past the end: clamped rows, never used)
+    __syncthreads();                  // A: tile t is in its slot; every wave is past PV / score write of tile t-1
+    if (wave == 0 && t == 0) STAMP(4);
     const unsigned char* slot = ring + (t % RSLOT) * SLOT;
     const int base = start + t * TN;
 
@@ -394,7 +416,7 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
       }
     }
   }
-  if (!NLOAD) ring_wait<0>();         // drain the clamped look-ahead loads before the workgroup's LDS is released
+  if (wave == 0) STAMP(6);
   if (SCORES) return;
 
   // ---- epilogue: normalise, write partial + lse --------------------------------------------------------------------
@@ -431,18 +453,14 @@ __global__ __launch_bounds__(256 + 64 * NLOAD) void latent_ring_kernel(const Rin
   }
 }
 
-#ifndef XKV_RING_NLOAD
-#define XKV_RING_NLOAD 2
-#endif
 template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE, int DVW = 512>
 static int launch_ring_t(const RingParams& p, int batch, hipStream_t st) {
   constexpr int SHM = RingShape<TN, DN, HAS_R, VMODE, NHB, DVW>::SHM;
-  constexpr int NLOAD = XKV_RING_NLOAD;
-  auto kern = latent_ring_kernel<T, TN, NHB, LO, DN, HAS_R, VMODE, DVW, NLOAD>;
+  auto kern = latent_ring_kernel<T, TN, NHB, LO, DN, HAS_R, VMODE, DVW>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SHM);
   if (e != hipSuccess) return (int)e;
   const int total = batch * p.groups * p.max_splits;
-  kern<<<dim3(xcd_grid(total, p.groups)), dim3(256 + 64 * NLOAD), SHM, st>>>(p);
+  kern<<<dim3(xcd_grid(total, p.groups)), dim3(512), SHM, st>>>(p);
   return launch_status();
 }
 
@@ -516,8 +534,6 @@ bool ring_eligible(const RingParams& p, bool vshared) {
   if (r && (p.dr != 64 || lo || vm != RING_VSHARED)) return false;
   if (p.sCl < p.dn || (r && p.sRl < 64) || (vm == RING_VDISTINCT && p.sVl < p.dv)) return false;
   if (vm == RING_VDISTINCT && p.dn == 512 && !lo && p.dv != 512) return false;
-  // the RoPE-key load addresses rows with a 32-bit byte offset from the sequence's first row
-  if (r && (int64_t)p.kv_len * p.sRl * 2 >= (int64_t)1 << 31) return false;
   return true;
 }
 
@@ -526,3 +542,9 @@ int launch_ring(const RingParams& p, int batch, bool vshared, int dtype, hipStre
 }
 
 }  // namespace xkv
+
+#ifdef XKV_RING_STAMPS
+extern "C" int xkv_debug_stamps(unsigned long long* host, int n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(xkv::ring_stamps), sizeof(unsigned long long) * n);
+}
+#endif
