@@ -46,9 +46,27 @@ def _quantiles(ts):
     return {"median": round(pick(0.5) * 1e3, 2), "p20": round(pick(0.2) * 1e3, 2), "p80": round(pick(0.8) * 1e3, 2)}
 
 
-def time_loop(fn, steps, warmup):
-    """`warmup` untimed calls, then exactly `steps` timed calls bracketed by synchronize.  Returns (total wall-clock ms,
-    per-step quantiles in us from HIP events recorded between the steps on the launch stream)."""
+SETTLE_S = 1.5
+
+
+def _settle(fn):
+    """Untimed calls of the workload about to be measured, for SETTLE_S seconds: a device that has idled (while the CPU
+    oracle ran, say) or has just run a different kernel needs tens of milliseconds of this load before it runs it at the
+    clock it sustains; until then every kernel is 4-10 % slower.  The --warmup steps still follow."""
+    t_end = time.perf_counter() + SETTLE_S
+    i = 0
+    while time.perf_counter() < t_end:
+        for _ in range(20):
+            fn(i)
+            i += 1
+        torch.cuda.synchronize()
+
+
+def time_loop(fn, steps, warmup, settle=True):
+    """Settling calls, `warmup` untimed calls, then exactly `steps` timed calls bracketed by synchronize.  Returns (total
+    wall-clock ms, per-step quantiles in us from HIP events recorded between the steps on the launch stream)."""
+    if settle:
+        _settle(fn)
     for i in range(warmup):
         fn(i)
     ev = _events(steps + 1)
@@ -63,8 +81,10 @@ def time_loop(fn, steps, warmup):
     return total, _quantiles([ev[i].elapsed_time(ev[i + 1]) for i in range(steps)])
 
 
-def time_kernel(fn, steps, warmup):
+def time_kernel(fn, steps, warmup, settle=True):
     """Average and median duration (ms) of one launch, HIP events recorded on the stream the kernel runs on."""
+    if settle:
+        _settle(fn)
     for i in range(warmup):
         fn(i)
     st, en = _events(steps), _events(steps)
@@ -174,17 +194,8 @@ def bench_c3(args, dev):
 
     first_ms = None
     if args.headline_first:   # diagnosis: the same loop as the first GPU work of the process
-        first_ms, _ = time_loop(step, args.steps, args.warmup)
-    # Bring the device to the clock it sustains under this load before anything is measured: in a process whose whole GPU
-    # life is a few tens of milliseconds every kernel - this one, the comparator, the copy kernels alike - runs 4-10 % slower
-    # than in steady state.  Untimed, reported as settle_s; the --warmup steps still precede the timed ones.
-    t_end = time.perf_counter() + args.settle
-    while time.perf_counter() < t_end:
-        for i in range(50):
-            step(i)
-        torch.cuda.synchronize()
-    # headline: exactly --steps layer steps after --warmup untimed ones, straight after the settling steps of the same workload
-    # (after a different kernel - the bandwidth-bound comparator, say - the first few dozen steps run ~7 % slower)
+        first_ms, _ = time_loop(step, args.steps, args.warmup, settle=False)
+    # headline: exactly --steps layer steps after the settling and --warmup steps of the same workload
     total_ms, step_q = time_loop(step, args.steps, args.warmup)
     us = total_ms * 1e3 / args.steps
     k_avg_ms, k_med_ms = time_kernel(stage1, max(args.steps, 50), max(args.warmup, 10))
@@ -228,7 +239,7 @@ def bench_c3(args, dev):
     res = {
         "metric": "us_per_layer_decode_step", "value": round(us, 2), "unit": "us",
         "higher_is_better": False,
-        "ms_per_step": total_ms / args.steps, "step_us": step_q, "settle_s": args.settle,
+        "ms_per_step": total_ms / args.steps, "step_us": step_q,
         "tokens_per_s": B / (us * 1e-6), "kv_tokens_scanned_per_s": B * L / (us * 1e-6),
         "config": {"workload": "c3 fused RoPE xKV decode: batch 16, 32q/8kv heads, d128, ctx %d, rank 512, "
                                "A shared by K/V and by a 4-layer group, per layer" % L, "kv_splits": S},
@@ -679,7 +690,8 @@ def main():
     ap.add_argument("--rank", type=int, default=192, help="rank of the qabrope workload (ropedecode: K rank, default 384)")
     ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16"], help="operand type of the qabrope workload")
     ap.add_argument("--settle", type=float, default=1.5,
-                    help="c3: seconds of untimed steps before any measurement (the device reaches its sustained clock)")
+                    help="seconds of untimed calls of a workload before each of its measurements (the device reaches the clock "
+                         "it sustains under that load); reported as settle_s")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-comparator", action="store_true")
     ap.add_argument("--headline-first", action="store_true",
@@ -695,6 +707,8 @@ def main():
     _lib.lib()  # fail loudly if the HIP library is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    global SETTLE_S
+    SETTLE_S = max(0.0, args.settle)
     if args.calib_copy:
         src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
@@ -711,6 +725,7 @@ def main():
             "higher_is_better": res.pop("higher_is_better"), "scaling": "weak", "vs_baseline": None,
             "dtype": "fp16" if (args.config == "pdsep" or (args.config == "qabrope" and args.dtype == "fp16")) else "bf16", "data": "synthetic"}
     line.update(res)
+    line["settle_s"] = args.settle
     line["device"] = device_info(dev)
     print(json.dumps(line))
 

@@ -64,7 +64,7 @@ __device__ unsigned long long ring_stamps[4096 * 8];
 #else
 #define STAMP(i)
 #endif
-constexpr int RING_QD = 2;      // tiles per loader wave in flight in registers (deeper queues only lengthen the start)
+constexpr int RING_QD = 2;      // tiles per loader wave in flight in registers (deeper queues only lengthen the start); >= 2
 enum { RING_SCORES = 0, RING_VSHARED = 1, RING_VDISTINCT = 2, RING_VHEADS = 3 };
 constexpr int RING_DVH = 128;   // head width of the per-head value rows (RING_VHEADS)
 
@@ -83,6 +83,12 @@ struct RingShape {
   static constexpr int TAIL = KSPLIT * HB * SP * 4 + HB * LDP * 2 + HB * 4 + HB * 8;
   static constexpr int RSLOT = 2;                          // the tile being read and the tile being written
   static constexpr int SHM = RSLOT * SLOT + TAIL;
+  // staging area of the query rows (no-PE features | RoPE features | pad; a second set for the low-order part); used when
+  // it fits beside the ring
+  static constexpr int QSTRIDE = (DN + (HAS_R ? 64 : 0)) * 2 + 16;
+  static constexpr int qst_bytes(bool lo) { return HB * QSTRIDE * (lo ? 2 : 1); }
+  static constexpr bool qst(bool lo) { return SHM + qst_bytes(lo) <= 160 * 1024; }
+  static constexpr int shm(bool lo) { return SHM + (qst(lo) ? qst_bytes(lo) : 0); }
   static_assert(SHM <= 160 * 1024, "ring does not fit the LDS");
 };
 
@@ -205,50 +211,109 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
       }
       if (HAS_R) st16(slot + CBYTES + iw * 1024, q[n]);
     };
+    // Iteration j: tile j - QD leaves the queue for the ring (its slot was released by barrier A of the tile before it) and
+    // tile j enters the queue in its place, so the look-ahead lives in the queue and a tile is waited for only when the
+    // next iteration needs it.  Every queue entry is loaded at one place in the code and stored at one place: the loads
+    // are invisible to the compiler, and a register copy between two such places would read a value that has not landed.
+    // Tiles past the end are fetched too (clamped rows, never used): the vmcnt arithmetic counts on QD - 1 younger tiles.
     if (wave == 4) STAMP(2);
-#pragma unroll
-    for (int d = 0; d < QD; ++d) {
-      fetch(d, rq[d]);
-      if (wave == 4 && d == 0) STAMP(5);
-    }
-    if (wave == 4) STAMP(7);
-    hand_on(0, rq[0]);                               // the ring starts empty
-    fetch(QD, rq[0]);
-    // During tile t the loader hands tile t+1 on (its slot was released by barrier A) and refills that queue entry: the
-    // look-ahead lives in the queue, a tile is waited for only when the next iteration needs it.
-    for (int t = 0; t < ntiles; t += QD) {          // t stays a multiple of QD, so every queue index below is static
+    for (int j0 = 0; j0 <= ntiles + QD; j0 += QD) {   // j0 stays a multiple of QD, so the queue index below is static
 #pragma unroll
       for (int u = 0; u < QD; ++u) {
-        if (t + u < ntiles) {
-          __syncthreads();                           // A: the slot of tile t+u-1 is free
-          hand_on(t + u + 1, rq[(u + 1) % QD]);
-          fetch(t + u + 1 + QD, rq[(u + 1) % QD]);
-          __syncthreads();                           // B
-          if (!SCORES) __syncthreads();              // C
+        const int j = j0 + u, k = j - QD;
+        if (j <= ntiles + QD) {
+          if (k >= 1) __syncthreads();                 // A of tile k-1: the slot of tile k-2 is free
+          if (k >= 0) hand_on(k, rq[u]);
+          fetch(j, rq[u]);
+          if (j == 0) {
+            if (wave == 4) STAMP(5);
+            __syncthreads();                           // start: the compute waves hold their query loads back until here
+          }
+          if (j == 1 && S::qst(LO)) __syncthreads();   // the compute waves' barrier between staging the query rows and reading them
+          if (k >= 1) {
+            __syncthreads();                           // B of tile k-1
+            if (!SCORES) __syncthreads();              // C of tile k-1
+          }
         }
       }
     }
     return;
   }
 
+  // The query loads of a workgroup are a burst several tiles long, and the CU serves its memory instructions in order: let
+  // the loaders put the first tiles ahead of it (they arrive at this barrier once those loads are issued).
+  __syncthreads();
   // ---- query operands in registers: lane (n16 = head row, g4) holds q[head][32 ks + 8 g4 .. +8] for its k-range ----
   vec8 qreg[KS_W][NHB], qlo[LO ? KS_W : 1][NHB];
   const int ks0 = kh * KS_W;
+  if constexpr (S::qst(LO)) {
+    // Whole rows, coalesced, each read once per workgroup, into the LDS; every lane then picks its operand pieces from there.
+    // (Read straight into the operand layout, a load instruction touches 16 half-used cache lines and two waves fetch
+    // the same rows: several microseconds at the start of a kernel that lasts tens.)
+    constexpr int QSTRIDE = S::QSTRIDE, RQ = HB / 4;   // wave w stages head rows RQ w .. +RQ
+    unsigned char* qst = smem + S::SHM;
+    u32x4 tmp[RQ * IPR * (LO ? 2 : 1) + (HAS_R ? 1 : 0)];
+    int n = 0;
 #pragma unroll
-  for (int hb = 0; hb < NHB; ++hb) {
-    int row = hb * 16 + n16;
-    row = row < hg ? row : hg - 1;   // head rows past the group repeat its last row: finite values that are never written out
-    const int64_t qh = (int64_t)b * p.hq + h0 + row;
-    const T* qn_l = reinterpret_cast<const T*>(p.qn) + qh * DN + ks0 * 32 + 8 * g4;
-    const T* ql_l = LO ? reinterpret_cast<const T*>(p.qn_lo) + qh * DN + ks0 * 32 + 8 * g4 : nullptr;
-    const T* qr_l = HAS_R ? reinterpret_cast<const T*>(p.qr) + qh * 64 + (ks0 - NKS_N) * 32 + 8 * g4 : nullptr;
+    for (int r = 0; r < RQ; ++r) {
+      int row = wave * RQ + r;
+      row = row < hg ? row : hg - 1;   // head rows past the group repeat its last row: finite values that are never written out
+      const int64_t qoff = ((int64_t)b * p.hq + h0 + row) * (DN * 2) + lane_off;
 #pragma unroll
-    for (int k = 0; k < KS_W; ++k) {
-      if (!HAS_R || ks0 + k < NKS_N) {
-        qreg[k][hb] = ld16<vec8>(qn_l + k * 32);
-        if (LO) qlo[k][hb] = ld16<vec8>(ql_l + k * 32);
-      } else {
-        qreg[k][hb] = ld16<vec8>(qr_l + k * 32);
+      for (int c = 0; c < IPR; ++c) {
+        if (!CPART || lane < DN / 8) {
+          tmp[n] = ld16<u32x4>(reinterpret_cast<const unsigned char*>(p.qn) + qoff + c * 1024);
+          if (LO) tmp[n + 1] = ld16<u32x4>(reinterpret_cast<const unsigned char*>(p.qn_lo) + qoff + c * 1024);
+        }
+        n += LO ? 2 : 1;
+      }
+    }
+    if (HAS_R && (lane >> 3) < RQ) {   // 128-byte RoPE rows: eight lanes each
+      int row = wave * RQ + (lane >> 3);
+      row = row < hg ? row : hg - 1;
+      tmp[n] = ld16<u32x4>(reinterpret_cast<const unsigned char*>(p.qr) + ((int64_t)b * p.hq + h0 + row) * 128 + (lane & 7) * 16);
+    }
+    n = 0;
+#pragma unroll
+    for (int r = 0; r < RQ; ++r) {
+      unsigned char* dst = qst + (wave * RQ + r) * QSTRIDE + lane_off;
+#pragma unroll
+      for (int c = 0; c < IPR; ++c) {
+        if (!CPART || lane < DN / 8) {
+          st16(dst + c * 1024, tmp[n]);
+          if (LO) st16(dst + HB * QSTRIDE + c * 1024, tmp[n + 1]);
+        }
+        n += LO ? 2 : 1;
+      }
+    }
+    if (HAS_R && (lane >> 3) < RQ) st16(qst + (wave * RQ + (lane >> 3)) * QSTRIDE + DN * 2 + (lane & 7) * 16, tmp[n]);
+    __syncthreads();
+#pragma unroll
+    for (int hb = 0; hb < NHB; ++hb) {
+      const unsigned char* src = qst + (hb * 16 + n16) * QSTRIDE + ks0 * 64 + g4 * 16;
+#pragma unroll
+      for (int k = 0; k < KS_W; ++k) {
+        qreg[k][hb] = ld16<vec8>(src + k * 64);
+        if (LO) qlo[k][hb] = ld16<vec8>(src + HB * QSTRIDE + k * 64);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int hb = 0; hb < NHB; ++hb) {
+      int row = hb * 16 + n16;
+      row = row < hg ? row : hg - 1;
+      const int64_t qh = (int64_t)b * p.hq + h0 + row;
+      const T* qn_l = reinterpret_cast<const T*>(p.qn) + qh * DN + ks0 * 32 + 8 * g4;
+      const T* ql_l = LO ? reinterpret_cast<const T*>(p.qn_lo) + qh * DN + ks0 * 32 + 8 * g4 : nullptr;
+      const T* qr_l = HAS_R ? reinterpret_cast<const T*>(p.qr) + qh * 64 + (ks0 - NKS_N) * 32 + 8 * g4 : nullptr;
+#pragma unroll
+      for (int k = 0; k < KS_W; ++k) {
+        if (!HAS_R || ks0 + k < NKS_N) {
+          qreg[k][hb] = ld16<vec8>(qn_l + k * 32);
+          if (LO) qlo[k][hb] = ld16<vec8>(ql_l + k * 32);
+        } else {
+          qreg[k][hb] = ld16<vec8>(qr_l + k * 32);
+        }
       }
     }
   }
@@ -455,7 +520,7 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
 
 template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE, int DVW = 512>
 static int launch_ring_t(const RingParams& p, int batch, hipStream_t st) {
-  constexpr int SHM = RingShape<TN, DN, HAS_R, VMODE, NHB, DVW>::SHM;
+  constexpr int SHM = RingShape<TN, DN, HAS_R, VMODE, NHB, DVW>::shm(LO);
   auto kern = latent_ring_kernel<T, TN, NHB, LO, DN, HAS_R, VMODE, DVW>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SHM);
   if (e != hipSuccess) return (int)e;
