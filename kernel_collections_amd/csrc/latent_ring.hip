@@ -532,10 +532,11 @@ static int launch_ring_t(const RingParams& p, int batch, hipStream_t st) {
 // which instantiation serves a call; -1: none (the register-staged kernel runs instead)
 // plain per-kv-head values [token][8 heads][128] under one shared, absorbed key basis: the call's kv groups all scan the
 // same C rows, so one workgroup per (sequence, split) serves every head
+// - or plain per-head keys too, viewed as one 1024-wide row against a block-diagonal query (no low-order part)
 static bool ring_vheads(const RingParams& p, bool vshared) {
+  const bool absorbed = p.qn_lo && (p.dn == 512 || p.dn == 384 || p.dn == 256), plain_keys = !p.qn_lo && p.dn == 1024;
   return !p.scores && !vshared && p.groups * RING_DVH == 1024 && p.dv == RING_DVH && p.sVh == RING_DVH && p.sCh == 0 &&
-         p.qn_lo && !p.R && p.hq <= 32 && p.hq % p.groups == 0 && (p.dn == 512 || p.dn == 384 || p.dn == 256) &&
-         p.sCl >= p.dn && p.sVl >= 1024;
+         (absorbed || plain_keys) && !p.R && p.hq <= 32 && p.hq % p.groups == 0 && p.sCl >= p.dn && p.sVl >= 1024;
 }
 
 static int ring_vmode(const RingParams& p, bool vshared) {
@@ -555,9 +556,12 @@ static int launch_ring_dt(const RingParams& p, int batch, bool vshared, hipStrea
     a.groups = 1;
     a.total_wg = batch * p.max_splits;
 #define XKV_RING_VH(NHB, DN) \
-  if ((p.hq <= 16 ? 1 : 2) == NHB && p.dn == DN) return launch_ring_t<T, 16, NHB, true, DN, false, RING_VHEADS, 1024>(a, batch, st);
+  if (lo && (p.hq <= 16 ? 1 : 2) == NHB && p.dn == DN) return launch_ring_t<T, 16, NHB, true, DN, false, RING_VHEADS, 1024>(a, batch, st);
     XKV_RING_VH(1, 512) XKV_RING_VH(2, 512) XKV_RING_VH(1, 384) XKV_RING_VH(2, 384) XKV_RING_VH(1, 256) XKV_RING_VH(2, 256)
 #undef XKV_RING_VH
+    if (p.dn == 1024 && !lo)
+      return p.hq <= 16 ? launch_ring_t<T, 16, 1, false, 1024, false, RING_VHEADS, 1024>(a, batch, st)
+                        : launch_ring_t<T, 16, 2, false, 1024, false, RING_VHEADS, 1024>(a, batch, st);
     return XKV_EUNSUPPORTED;
   }
   const int nhb = hg <= 16 ? 1 : 2;

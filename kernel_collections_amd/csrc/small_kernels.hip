@@ -360,8 +360,11 @@ static int launch_merge(const float* partial, const float* lse, void* out, const
                         int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, float* lse_out, int64_t sLb, int64_t sLh,
                         int split_cap, hipStream_t st) {
   // few splits: one workgroup per kv head (vB read once for its heads); many splits: one per query head, so that the
-  // partial rows of a long sequence are spread over more CUs
-  const int hpw = (max_splits > 16 || hq / hkv > 16) ? 1 : hq / hkv;
+  // partial rows of a long sequence are spread over more CUs - unless the kv heads alone fill half the device and there
+  // is an up-projection, whose vB rows then weigh more than the partial rows
+  const int g = hq / hkv;
+  const bool enough_wgs = vB && (int64_t)hkv * batch >= 128;   // vB costs more than the partial rows: keep it read once per kv head
+  const int hpw = (g > 16 || (max_splits > 16 && !enough_wgs)) ? 1 : g;
   size_t shm = (size_t)hpw * (dv + max_splits) * sizeof(float);
   // a small grid over many splits is bound by the latency of its partial-row loads: split the up-projection's columns
   // over more workgroups

@@ -48,13 +48,23 @@ def decode_attention_fwd(q, k_buffer, v_buffer, o, num_kv_splits, max_kv_splits,
     kv_len = k_buffer.shape[1]
     q3 = ops._q3(q)
     k_buffer, v_buffer = ops.as_rows(k_buffer), ops.as_rows(v_buffer)
-    cap = MAX_SPLIT_TOKENS
+    # 8 kv heads of 128: one workgroup serves every head of a split - a token's keys are one 1024-wide row against a
+    # block-diagonal query, its values one 1024-wide row of per-head pieces - so whole 2 KiB rows stream through the LDS ring
+    wide = (hkv * d == 1024 and d == 128 and hq <= 32 and k_buffer.stride(2) == d and v_buffer.stride(2) == d
+            and k_buffer.stride(1) >= 1024 and v_buffer.stride(1) >= 1024)
+    cap = MAX_SPLIT_TOKENS_WIDE if wide else MAX_SPLIT_TOKENS
     S = ops.capped_splits(kv_len, S, cap)     # room in the workspaces for the splits the kernels may add (host arithmetic only)
     partial, lse = ops.workspaces(batch, hq, S, dv, q.device)
-    ops.latent_stage1(q3, None, None,
-                      (k_buffer, k_buffer.stride(0), k_buffer.stride(1), k_buffer.stride(2), d), None,
-                      (v_buffer, v_buffer.stride(0), v_buffer.stride(1), v_buffer.stride(2), dv),
-                      partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale), split_cap=cap)
+    if wide:
+        ops.latent_stage1(ops.blockdiag_q(q3, hkv), None, None,
+                          (k_buffer, k_buffer.stride(0), k_buffer.stride(1), 0, hkv * d), None,
+                          (v_buffer, v_buffer.stride(0), v_buffer.stride(1), v_buffer.stride(2), dv),
+                          partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale), split_cap=cap)
+    else:
+        ops.latent_stage1(q3, None, None,
+                          (k_buffer, k_buffer.stride(0), k_buffer.stride(1), k_buffer.stride(2), d), None,
+                          (v_buffer, v_buffer.stride(0), v_buffer.stride(1), v_buffer.stride(2), dv),
+                          partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale), split_cap=cap)
     return ops.merge_stage2(partial, lse, o, None, splits, lens, batch, hq, hq, kv_len, S, split_cap=cap)
 
 
