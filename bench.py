@@ -481,7 +481,9 @@ def bench_c4(args, dev, vfact):
         gqa.MAX_SPLIT_TOKENS, gqa.MAX_SPLIT_TOKENS_WIDE = saved
     algo_bytes = sum(lens) * per_tok
     gbs = algo_bytes / (us * 1e-6) / 1e9
-    limit = gqa.MAX_SPLIT_TOKENS_WIDE if vfact else gqa.MAX_SPLIT_TOKENS
+    # the split length the wrappers planned on the device for this batch (read back here, outside every timed region)
+    plan_S = ops.capped_splits(Lmax, S, gqa.MAX_SPLIT_TOKENS_WIDE)
+    limit = int(ops.plan_splits(kl, ns, plan_S, gqa.MAX_SPLIT_TOKENS_WIDE, ops.num_cus())[0].item())
     cpu = None
     if not args.no_cpu:
         # an eighth of every length (fp32): the scan is linear in the number of tokens, value = time x 8
@@ -506,8 +508,10 @@ def bench_c4(args, dev, vfact):
         "config": {"workload": "c4 ragged split-K GQA%s: batch 32, lens log-uniform [1024,131072], %d-token splits at the call"
                                % (" V-factorised r512" if vfact else "", split), "sum_len": sum(lens), "max_len": Lmax,
                    "kv_splits_max_at_the_call": S,
-                   "kv_splits_max_in_the_kernel": max(S, -(-Lmax // limit)) if limit and Lmax > S * limit else S,
-                   "longest_split_in_the_kernel_tokens": min(split, limit) if limit else split},
+                   "split_length_planned_on_the_device_tokens": limit,
+                   "kv_splits_max_in_the_kernel": max(max(s_, -(-n // limit)) for n, s_ in zip(lens, ns_l)),
+                   "workgroups_with_work": sum(max(s_, -(-n // limit)) for n, s_ in zip(lens, ns_l)),
+                   "compute_units": ops.num_cus()},
         "roofline": {"bound": "hbm", "kernel": "latent_ring_kernel" if vfact else "latent_stage1_kernel",
                      "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None,

@@ -23,6 +23,11 @@
  *     the device by stage 1 and by the merge alike, so a ragged batch whose caller asks for long splits is still spread over
  *     the whole chip.  max_splits - the split dimension of the workspaces - must then be at least ceil(kv_len /
  *     split_cap_tokens) (XKV_EINVAL otherwise).  Split-K is exact under the merge: the result does not depend on it.
+ *   - `split_plan` (same two entry points; NULL = off): the int32 array xkv_plan_splits wrote in device memory.  Its
+ *     first word is a cap; the cap in force is then max(split_cap_tokens, plan[0]) - the host value bounds the workspaces,
+ *     the device value, chosen from the lengths of the batch, which the host never reads, makes the splits as long as the
+ *     batch allows while every CU still gets one.  Stage 1 also takes its (sequence, split) pairs from the plan's job
+ *     list, so the workgroups that have work are the first ones of the grid and spread evenly over the XCDs.
  */
 #ifndef XKV_HIP_H
 #define XKV_HIP_H
@@ -33,7 +38,7 @@
 extern "C" {
 #endif
 
-#define XKV_ABI_VERSION 4
+#define XKV_ABI_VERSION 5
 
 enum { XKV_F16 = 0, XKV_BF16 = 1, XKV_F32 = 2 };
 
@@ -131,7 +136,7 @@ int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_operand qr,
                       void* scores_out, int scores_dtype,
                       const int32_t* num_kv_splits, const int32_t* kv_lens,
                       int batch, int hq, int n_kv_groups, int kv_len, int max_splits, int split_cap_tokens,
-                      float sm_scale, float logit_cap, int dtype, void* stream);
+                      const int32_t* split_plan, float sm_scale, float logit_cap, int dtype, void* stream);
 
 /* Split-K stage 1 with fused key reconstruction and RoPE:
  *
@@ -207,9 +212,23 @@ int xkv_merge_stage2(const float* partial, const float* lse, void* out,
                      const void* vB, int64_t stride_vB_b, int64_t stride_vB_h, int64_t stride_vB_r,
                      int d_out, int vB_dtype,
                      const int32_t* num_kv_splits, const int32_t* kv_lens,
-                     int batch, int hq, int hkv, int kv_len, int max_splits, int split_cap_tokens, int dv,
+                     int batch, int hq, int hkv, int kv_len, int max_splits, int split_cap_tokens,
+                     const int32_t* split_plan, int dv,
                      int64_t stride_o_b, int64_t stride_o_h, int out_dtype,
                      float* lse_out, int64_t stride_lse_b, int64_t stride_lse_h, void* stream);
+
+/* Split plan for a ragged batch: plan[0] = cap, the smallest multiple of 32, not below floor_tokens, such that
+ * sum_b ceil(kv_lens[b] / cap) <= target_jobs; plan[1] = the number of jobs, i.e. live (sequence, split) pairs when
+ * sequence b is cut into max(num_kv_splits[b], ceil(kv_lens[b] / cap)) splits; plan[2 + 2 j], plan[3 + 2 j] = sequence and
+ * split of job j (whole splits first, each sequence's last - shorter - split after them).  With target_jobs = the number
+ * of CUs, a stage 1 that runs one workgroup per CU gives every CU exactly one job and the jobs are as equal as the lengths
+ * allow; a batch scanned in fixed-length splits ends on whatever the last workgroups happen to hold.  plan holds
+ * 2 + 2 * batch * max_splits int32 (max_splits as passed to stage 1, >= ceil(kv_len / floor_tokens)).  Pass plan as
+ * split_plan, and floor_tokens as split_cap_tokens, to xkv_latent_stage1 and xkv_merge_stage2 on the same stream.  One
+ * small workgroup; no host synchronisation.  No counterpart in the reference, whose batches have one length
+ * (flash_decoding/gqa.py:60,194). */
+int xkv_plan_splits(const int32_t* kv_lens, const int32_t* num_kv_splits, int batch, int max_splits, int floor_tokens,
+                    int target_jobs, int32_t* plan, void* stream);
 
 /* Measurement aids (no counterpart in the reference; bench.py --config ceilings): what this GPU sustains with nothing but
  * the instruction a kernel is bound by.

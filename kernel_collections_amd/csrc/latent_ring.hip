@@ -97,8 +97,10 @@ struct RingShape {
 // DN features of the C row / V is a second, DVW-wide row stream / V is a second stream of DVW / 128 per-kv-head value
 // rows of 128 features (plain values under absorbed factorised keys): the workgroup serves every query head, wave w
 // accumulates kv heads 2w, 2w+1, and query head h multiplies the values of kv head h / (heads per kv head).
+// DN 1024 means eight plain kv heads of 128 side by side in a token row, against compact query rows [b, hq, 128].
 template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE, int DVW>
 __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
+  static_assert(DN != 1024 || (!LO && !HAS_R), "the 1024-wide form is plain per-head keys");
   typedef typename Elem<T>::vec8 vec8;
   typedef RingShape<TN, DN, HAS_R, VMODE, NHB, DVW> S;
   constexpr bool SCORES = VMODE == RING_SCORES, V2 = VMODE >= RING_VDISTINCT, VHEADS = VMODE == RING_VHEADS;
@@ -136,11 +138,17 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
   const int wg = xcd_cluster_remap(blockIdx.x, p.groups);   // the kv groups of one (sequence, split) share an L2
   if (wg >= p.total_wg) return;
   const int group = wg % p.groups;
-  const int split = (wg / p.groups) % p.max_splits;
-  const int b = wg / (p.groups * p.max_splits);
+  int split = (wg / p.groups) % p.max_splits;
+  int b = wg / (p.groups * p.max_splits);
+  if (p.split_plan) {   // job list: the live (sequence, split) pairs come first in the grid
+    const int job = wg / p.groups;
+    if (job >= p.split_plan[1]) return;
+    b = p.split_plan[2 + 2 * job];
+    split = p.split_plan[3 + 2 * job];
+  }
   const int L = p.kv_lens ? p.kv_lens[b] : p.kv_len;
   int start, end;
-  split_bounds(L, effective_splits(L, p.num_splits[b], p.split_cap), split, start, end);
+  split_bounds(L, effective_splits(L, p.num_splits[b], split_cap_in_force(p.split_cap, p.split_plan)), split, start, end);
   if (end <= start) return;
   const int hg = p.hq / p.groups, h0 = group * hg;
   const int ntiles = (end - start + TN - 1) / TN;
@@ -295,6 +303,24 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
       for (int k = 0; k < KS_W; ++k) {
         qreg[k][hb] = ld16<vec8>(src + k * 64);
         if (LO) qlo[k][hb] = ld16<vec8>(src + HB * QSTRIDE + k * 64);
+      }
+    }
+  } else if constexpr (DN == 1024) {
+    // Eight kv heads of 128 side by side in a token row: the query is block-diagonal and comes as its compact rows
+    // [b, hq, 128]; head row r multiplies only k-steps 4 kvh .. 4 kvh + 3 of its kv head kvh = r / (heads per kv head).
+    const int hpq = hg / 8;
+#pragma unroll
+    for (int hb = 0; hb < NHB; ++hb) {
+      int row = hb * 16 + n16;
+      row = row < hg ? row : hg - 1;
+      const int kvh = row / hpq;
+      const T* ql = reinterpret_cast<const T*>(p.qn) + ((int64_t)b * p.hq + h0 + row) * 128 + 8 * g4;
+#pragma unroll
+      for (int k = 0; k < KS_W; ++k) {
+        const int ks = ks0 + k;
+        vec8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if ((ks >> 2) == kvh) v = ld16<vec8>(ql + (ks & 3) * 32);
+        qreg[k][hb] = v;
       }
     }
   } else {
@@ -534,7 +560,8 @@ static int launch_ring_t(const RingParams& p, int batch, hipStream_t st) {
 // same C rows, so one workgroup per (sequence, split) serves every head
 // - or plain per-head keys too, viewed as one 1024-wide row against a block-diagonal query (no low-order part)
 static bool ring_vheads(const RingParams& p, bool vshared) {
-  const bool absorbed = p.qn_lo && (p.dn == 512 || p.dn == 384 || p.dn == 256), plain_keys = !p.qn_lo && p.dn == 1024;
+  const bool absorbed = p.qn_lo && (p.dn == 512 || p.dn == 384 || p.dn == 256);
+  const bool plain_keys = !p.qn_lo && p.dn == 1024 && p.heads_in_row == 8;
   return !p.scores && !vshared && p.groups * RING_DVH == 1024 && p.dv == RING_DVH && p.sVh == RING_DVH && p.sCh == 0 &&
          (absorbed || plain_keys) && !p.R && p.hq <= 32 && p.hq % p.groups == 0 && p.sCl >= p.dn && p.sVl >= 1024;
 }
@@ -599,6 +626,7 @@ bool ring_eligible(const RingParams& p, bool vshared) {
   const bool lo = p.qn_lo != nullptr, r = p.R != nullptr;
   if (vm == RING_VHEADS) return true;
   if (hg > 32 || vm < 0) return false;
+  if ((p.dn == 1024) != (p.heads_in_row == 8)) return false;   // the 1024-wide form is only the eight-heads-in-a-row one
   if (p.dn != 512 && !(p.dn == 1024 && vm == RING_VDISTINCT && !lo) && !((p.dn == 384 || p.dn == 256) && lo && !r)) return false;
   if (r && (p.dr != 64 || lo || vm != RING_VSHARED)) return false;
   if (p.sCl < p.dn || (r && p.sRl < 64) || (vm == RING_VDISTINCT && p.sVl < p.dv)) return false;

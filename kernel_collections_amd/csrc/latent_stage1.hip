@@ -50,12 +50,18 @@ __global__ __launch_bounds__(256) void latent_stage1_kernel(const LatentParams p
   const int wg = xcd_cluster_remap(blockIdx.x, p.groups);   // the kv groups of one (sequence, split) share an L2
   if (wg >= p.total_wg) return;
   const int group = wg % p.groups;
-  const int split = (wg / p.groups) % p.max_splits;
-  const int b = wg / (p.groups * p.max_splits);
+  int split = (wg / p.groups) % p.max_splits;
+  int b = wg / (p.groups * p.max_splits);
+  if (p.split_plan) {   // job list: the live (sequence, split) pairs come first in the grid
+    const int job = wg / p.groups;
+    if (job >= p.split_plan[1]) return;
+    b = p.split_plan[2 + 2 * job];
+    split = p.split_plan[3 + 2 * job];
+  }
 
   const int L = p.kv_lens ? p.kv_lens[b] : p.kv_len;
   int start, end;
-  split_bounds(L, effective_splits(L, p.num_splits[b], p.split_cap), split, start, end);
+  split_bounds(L, effective_splits(L, p.num_splits[b], split_cap_in_force(p.split_cap, p.split_plan)), split, start, end);
   if (end <= start) return;
 
   const int hg = p.hq / p.groups;  // heads of this kv group
@@ -357,7 +363,8 @@ static bool ptr16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) 
 extern "C" int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_operand qr, xkv_kv_operand C,
                                  xkv_kv_operand R, xkv_kv_operand V, float* partial, float* lse, void* scores_out,
                                  int scores_dtype, const int32_t* num_kv_splits, const int32_t* kv_lens, int batch,
-                                 int hq, int n_kv_groups, int kv_len, int max_splits, int split_cap_tokens, float sm_scale,
+                                 int hq, int n_kv_groups, int kv_len, int max_splits, int split_cap_tokens,
+                                 const int32_t* split_plan, float sm_scale,
                                  float logit_cap,
                                  int dtype, void* stream) {
   if (!qn.ptr || !C.ptr || !num_kv_splits || batch <= 0 || hq <= 0 || n_kv_groups <= 0 || kv_len <= 0 ||
@@ -365,6 +372,7 @@ extern "C" int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_oper
     return XKV_EINVAL;
   // with a cap the longest sequence may need cdiv(kv_len, cap) splits: the workspace must have a row for each
   if (split_cap_tokens < 0 || (split_cap_tokens > 0 && max_splits < cdiv(kv_len, split_cap_tokens))) return XKV_EINVAL;
+  if (split_plan && split_cap_tokens <= 0) return XKV_EINVAL;   // the host value is what bounds the workspaces
   const bool scores_only = scores_out != nullptr;
   if (!scores_only && (!V.ptr || !partial || !lse)) return XKV_EINVAL;
   if (dtype != XKV_BF16 && dtype != XKV_F16) return XKV_EDTYPE;
@@ -395,11 +403,28 @@ extern "C" int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_oper
   p.partial = partial; p.lse = lse; p.scores = scores_out; p.scores_dtype = scores_dtype;
   p.num_splits = num_kv_splits; p.kv_lens = kv_lens;
   p.hq = hq; p.groups = n_kv_groups; p.kv_len = kv_len; p.max_splits = max_splits; p.split_cap = split_cap_tokens;
+  p.split_plan = split_plan;
   p.total_wg = batch * n_kv_groups * max_splits;
   p.sm_scale = sm_scale; p.logit_cap = logit_cap;
+  p.heads_in_row = 0;
   const bool vshared = !scores_only && V.ptr == C.ptr && V.stride_b == C.stride_b && V.stride_l == C.stride_l &&
                        V.stride_h == C.stride_h && V.dim == C.dim;
   hipStream_t st = (hipStream_t)stream;
+  // Plain keys of 8 kv heads x 128 side by side in a token row, values either laid out the same way or one shared
+  // 256 .. 512-wide row (V = v_A): one workgroup serves every head of a split.  A token's keys are then one 1024-wide row
+  // against a block-diagonal query (which the kernel builds from the compact rows), so whole 2 KiB rows stream through
+  // the LDS ring and the shared value row is read once per token instead of once per kv head.
+  if (!scores_only && !qn_lo && !dr && C.dim == 128 && n_kv_groups == 8 && C.stride_h == 128 && C.stride_l >= 1024 &&
+      hq <= 32) {
+    const bool v_heads = V.dim == 128 && V.stride_h == 128 && V.stride_l >= 1024;
+    const bool v_shared_row = V.stride_h == 0 && (V.dim == 256 || V.dim == 384 || V.dim == 512) && V.stride_l >= V.dim;
+    if (v_heads || v_shared_row) {
+      LatentParams w = p;
+      w.dn = 1024; w.sCh = 0; w.heads_in_row = 8;
+      if (v_shared_row) { w.groups = 1; w.total_wg = batch * max_splits; }
+      if (ring_eligible(w, false)) return launch_ring(w, batch, false, dtype, st);
+    }
+  }
   if (ring_eligible(p, vshared)) return launch_ring(p, batch, vshared, dtype, st);
   if (dtype == XKV_BF16)
     return hg <= 16 ? dispatch_latent<__bf16, 1>(p, batch, vshared, st) : dispatch_latent<__bf16, 2>(p, batch, vshared, st);

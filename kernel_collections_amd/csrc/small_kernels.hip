@@ -176,7 +176,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     const TB* __restrict__ vB, int64_t sVb, int64_t sVh, int64_t sVr, int d_out,
     const int32_t* __restrict__ num_kv_splits, const int32_t* __restrict__ kv_lens,
     int hq, int hkv, int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, int hpw,
-    float* __restrict__ lse_out, int64_t sLb, int64_t sLh, int d_blk, int split_cap) {
+    float* __restrict__ lse_out, int64_t sLb, int64_t sLh, int d_blk, int split_cap, const int32_t* __restrict__ split_plan) {
   extern __shared__ float merged[];  // [G][dv], then the split weights [G][max_splits]
   __shared__ float fin[4 * 512];     // per-head-block totals of the up-projection
   // this workgroup: heads hfirst .. hfirst + G - 1 of sequence b, all of kv head kh (G = hpw divides the GQA group size)
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     d_out = d_blk;
   }
   const int L = kv_lens ? kv_lens[b] : kv_len;
-  const int ns = effective_splits(L, num_kv_splits[b], split_cap);
+  const int ns = effective_splits(L, num_kv_splits[b], split_cap_in_force(split_cap, split_plan));
   float* wts = merged + G * dv;
   int nlive = 0;
   {
@@ -358,7 +358,7 @@ template <typename O, typename TB>
 static int launch_merge(const float* partial, const float* lse, void* out, const void* vB, int64_t sVb, int64_t sVh,
                         int64_t sVr, int d_out, const int32_t* ns, const int32_t* kl, int batch, int hq, int hkv,
                         int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, float* lse_out, int64_t sLb, int64_t sLh,
-                        int split_cap, hipStream_t st) {
+                        int split_cap, const int32_t* split_plan, hipStream_t st) {
   // few splits: one workgroup per kv head (vB read once for its heads); many splits: one per query head, so that the
   // partial rows of a long sequence are spread over more CUs - unless the kv heads alone fill half the device and there
   // is an up-projection, whose vB rows then weigh more than the partial rows
@@ -372,13 +372,101 @@ static int launch_merge(const float* partial, const float* lse, void* out, const
   if (vB && (hq / hpw) * batch < 128 && max_splits >= 64 && d_out % 32 == 0) zb = d_out >= 512 ? 4 : d_out >= 256 ? 2 : 1;
   merge_stage2_kernel<O, TB><<<dim3(hq / hpw, batch, zb), dim3(256), shm, st>>>(partial, lse, (O*)out, (const TB*)vB, sVb, sVh,
                                                                                sVr, d_out, ns, kl, hq, hkv, kv_len, max_splits,
-                                                                               dv, sOb, sOh, hpw, lse_out, sLb, sLh, d_out / zb, split_cap);
+                                                                               dv, sOb, sOh, hpw, lse_out, sLb, sLh, d_out / zb, split_cap, split_plan);
   return launch_status();
+}
+
+// plan[0]: smallest multiple of 32 >= floor_tokens with sum_b ceil(len_b / cap) <= target_jobs, by bisection over cap / 32
+// (the job count falls monotonically as the cap grows).  Then the job list: sequence b has n_b = effective_splits(len_b,
+// num_splits[b], cap) splits of which the live ones are a prefix; whole splits first (sequence-major), every sequence's last
+// live split - the short one - after them.  One workgroup; thread t handles sequences t, t + 256, ...
+__global__ __launch_bounds__(256) void plan_splits_kernel(const int32_t* __restrict__ kv_lens, const int32_t* __restrict__ num_splits,
+                                                          int batch, int max_splits, int floor_tokens, int target_jobs,
+                                                          int32_t* __restrict__ plan) {
+  __shared__ int red[4];
+  __shared__ int carry;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  auto block_reduce = [&](int v, bool take_max) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int w = __shfl_xor(v, o);
+      v = take_max ? (w > v ? w : v) : v + w;
+    }
+    __syncthreads();            // red is free again
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    int r = red[0];
+#pragma unroll
+    for (int i = 1; i < 4; ++i) r = take_max ? (red[i] > r ? red[i] : r) : r + red[i];
+    return r;
+  };
+  int lm = 0;
+  for (int b = threadIdx.x; b < batch; b += 256) lm = kv_lens[b] > lm ? kv_lens[b] : lm;
+  lm = block_reduce(lm, true);
+  int lo = cdiv(floor_tokens > 32 ? floor_tokens : 32, 32), hi = cdiv(lm > 32 ? lm : 32, 32);   // in units of 32 tokens
+  if (hi < lo) hi = lo;
+  while (lo < hi) {   // if even one job per sequence is too many, this ends on the longest length
+    const int mid = (lo + hi) >> 1, cap = mid * 32;
+    int jobs = 0;
+    for (int b = threadIdx.x; b < batch; b += 256) jobs += cdiv(kv_lens[b] > 0 ? kv_lens[b] : 0, cap);
+    jobs = block_reduce(jobs, false);
+    if (jobs <= target_jobs) hi = mid; else lo = mid + 1;
+  }
+  const int cap = lo * 32;
+  // live splits of a sequence, in the arithmetic of split_bounds
+  auto live_of = [&](int b) {
+    const int L = kv_lens[b];
+    if (L <= 0) return 0;
+    const int n = effective_splits(L, num_splits[b], cap);
+    const int per = cdiv(cdiv(L, n), MIN_BLOCK_KV) * MIN_BLOCK_KV;
+    const int live = cdiv(L, per);
+    return live < max_splits ? live : max_splits;
+  };
+  // exclusive prefix sums over the sequences, 256 at a time: first of (live - 1) whole splits, then of the last splits
+  if (threadIdx.x == 0) carry = 0;
+  __syncthreads();
+  for (int pass = 0; pass < 2; ++pass) {
+    for (int b0 = 0; b0 < batch; b0 += 256) {
+      const int b = b0 + threadIdx.x;
+      const int live = b < batch ? live_of(b) : 0;
+      const int mine = pass == 0 ? (live > 0 ? live - 1 : 0) : (live > 0 ? 1 : 0);
+      // inclusive scan within the wave, then across the four waves
+      int incl = mine;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int w = __shfl_up(incl, o);
+        if (lane >= o) incl += w;
+      }
+      __syncthreads();
+      if (lane == 63) red[wave] = incl;
+      __syncthreads();
+      int before = carry;
+      for (int i = 0; i < wave; ++i) before += red[i];
+      const int start = before + incl - mine;
+      if (pass == 0) {
+        for (int s2 = 0; s2 < mine; ++s2) { plan[2 + 2 * (start + s2)] = b; plan[3 + 2 * (start + s2)] = s2; }
+      } else if (mine) {
+        plan[2 + 2 * start] = b; plan[3 + 2 * start] = live - 1;
+      }
+      __syncthreads();
+      if (threadIdx.x == 255) carry = start + mine;
+      __syncthreads();
+    }
+  }
+  if (threadIdx.x == 0) { plan[0] = cap; plan[1] = carry; }
 }
 
 }  // namespace xkv
 
 using namespace xkv;
+
+extern "C" int xkv_plan_splits(const int32_t* kv_lens, const int32_t* num_kv_splits, int batch, int max_splits, int floor_tokens,
+                               int target_jobs, int32_t* plan, void* stream) {
+  if (!kv_lens || !num_kv_splits || !plan || batch <= 0 || max_splits <= 0 || floor_tokens <= 0 || target_jobs <= 0) return XKV_EINVAL;
+  plan_splits_kernel<<<dim3(1), dim3(256), 0, (hipStream_t)stream>>>(kv_lens, num_kv_splits, batch, max_splits, floor_tokens,
+                                                                     target_jobs, plan);
+  return launch_status();
+}
 
 extern "C" int xkv_abi_version(void) { return XKV_ABI_VERSION; }
 
@@ -480,16 +568,17 @@ extern "C" int xkv_blockdiag_q(const void* q, void* out, int batch, int hq, int 
 extern "C" int xkv_merge_stage2(const float* partial, const float* lse, void* out, const void* vB, int64_t sVb,
                                 int64_t sVh, int64_t sVr, int d_out, int vB_dtype, const int32_t* ns,
                                 const int32_t* kl, int batch, int hq, int hkv, int kv_len, int max_splits,
-                                int split_cap_tokens, int dv, int64_t sOb, int64_t sOh, int out_dtype, float* lse_out,
+                                int split_cap_tokens, const int32_t* split_plan, int dv, int64_t sOb, int64_t sOh, int out_dtype, float* lse_out,
                                 int64_t sLb, int64_t sLh, void* stream) {
   if (!partial || !lse || !out || !ns || batch <= 0 || hq <= 0 || hkv <= 0 || max_splits <= 0 || dv <= 0)
     return XKV_EINVAL;
   if (split_cap_tokens < 0 || (split_cap_tokens > 0 && (kv_len <= 0 || max_splits < cdiv(kv_len, split_cap_tokens)))) return XKV_EINVAL;
+  if (split_plan && split_cap_tokens <= 0) return XKV_EINVAL;
   if (hq % hkv || hq / hkv > 32 || dv > 512) return XKV_EUNSUPPORTED;
   if (vB && (d_out <= 0 || d_out > 512 || d_out % 8)) return XKV_EUNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
 #define XKV_MERGE(O, TB) \
-  return launch_merge<O, TB>(partial, lse, out, vB, sVb, sVh, sVr, d_out, ns, kl, batch, hq, hkv, kv_len, max_splits, dv, sOb, sOh, lse_out, sLb, sLh, split_cap_tokens, st)
+  return launch_merge<O, TB>(partial, lse, out, vB, sVb, sVh, sVr, d_out, ns, kl, batch, hq, hkv, kv_len, max_splits, dv, sOb, sOh, lse_out, sLb, sLh, split_cap_tokens, split_plan, st)
   const int bt = vB ? vB_dtype : XKV_BF16;
   if (bt != XKV_BF16 && bt != XKV_F16) return XKV_EDTYPE;
   switch (out_dtype) {

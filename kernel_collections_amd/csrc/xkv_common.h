@@ -85,6 +85,13 @@ __host__ __device__ __forceinline__ int effective_splits(int kv_len, int num_spl
   return num_splits;
 }
 
+// The cap in force: the host's value, raised by the one a planning kernel left in the first word of its plan (if any).
+__device__ __forceinline__ int split_cap_in_force(int cap_tokens, const int32_t* plan) {
+  if (!plan) return cap_tokens;
+  const int d = plan[0];
+  return d > cap_tokens ? d : cap_tokens;
+}
+
 // Reductions over the 4 lane groups {n, n+16, n+32, n+48} that share a column
 // index in the 16x16 MFMA result layout.
 __device__ __forceinline__ float group4_max(float v) {

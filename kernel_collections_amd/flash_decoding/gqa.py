@@ -20,7 +20,25 @@ from kernel_collections_amd import ops
 # split-K is exact under the merge, so the caller's count is a lower bound on the parallelism, not part of the result, and a
 # ragged batch scanned in 4096-token splits would otherwise leave most CUs idle behind its longest sequences.
 MAX_SPLIT_TOKENS = 1024
-MAX_SPLIT_TOKENS_WIDE = 2048   # the all-heads form of decode_attention_fwd_v_factorized (one workgroup serves 32 heads)
+# The all-heads ("wide") forms run one workgroup per CU and per (sequence, split), hkv times fewer workgroups than the
+# per-head form.  There the split length is planned per call: the shortest that still cuts the batch into at most one split
+# per CU, so that every CU gets one job and the jobs are as equal as the lengths allow - never below this floor, which is
+# also what sizes the workspaces (0: the caller's splits as they are).
+MAX_SPLIT_TOKENS_WIDE = 1024
+
+
+def _plan_wide(lens, splits, S, batch, kv_len):
+    """(cap that sizes the workspaces, their split dimension, split plan on the device or None) of an all-heads call."""
+    floor = MAX_SPLIT_TOKENS_WIDE
+    if not floor:
+        return 0, S, None
+    jobs = ops.num_cus()
+    if lens is None:      # one length: plain host arithmetic
+        per_seq = max(1, jobs // batch)
+        cap = max(floor, -(-(-(-kv_len // per_seq)) // 32) * 32)
+        return cap, ops.capped_splits(kv_len, S, cap), None
+    S = ops.capped_splits(kv_len, S, floor)
+    return floor, S, ops.plan_splits(lens, splits, S, floor, jobs)
 
 
 def _prep(q, k_buffer, num_kv_splits, max_kv_splits, kv_lens):
@@ -48,24 +66,21 @@ def decode_attention_fwd(q, k_buffer, v_buffer, o, num_kv_splits, max_kv_splits,
     kv_len = k_buffer.shape[1]
     q3 = ops._q3(q)
     k_buffer, v_buffer = ops.as_rows(k_buffer), ops.as_rows(v_buffer)
-    # 8 kv heads of 128: one workgroup serves every head of a split - a token's keys are one 1024-wide row against a
-    # block-diagonal query, its values one 1024-wide row of per-head pieces - so whole 2 KiB rows stream through the LDS ring
+    # 8 kv heads of 128 side by side in a token row: stage 1 serves every head of a split from one workgroup (whole 2 KiB
+    # rows through its LDS ring), so there are hkv times fewer workgroups and a split may be twice as long
     wide = (hkv * d == 1024 and d == 128 and hq <= 32 and k_buffer.stride(2) == d and v_buffer.stride(2) == d
             and k_buffer.stride(1) >= 1024 and v_buffer.stride(1) >= 1024)
-    cap = MAX_SPLIT_TOKENS_WIDE if wide else MAX_SPLIT_TOKENS
-    S = ops.capped_splits(kv_len, S, cap)     # room in the workspaces for the splits the kernels may add (host arithmetic only)
-    partial, lse = ops.workspaces(batch, hq, S, dv, q.device)
     if wide:
-        ops.latent_stage1(ops.blockdiag_q(q3, hkv), None, None,
-                          (k_buffer, k_buffer.stride(0), k_buffer.stride(1), 0, hkv * d), None,
-                          (v_buffer, v_buffer.stride(0), v_buffer.stride(1), v_buffer.stride(2), dv),
-                          partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale), split_cap=cap)
-    else:
-        ops.latent_stage1(q3, None, None,
-                          (k_buffer, k_buffer.stride(0), k_buffer.stride(1), k_buffer.stride(2), d), None,
-                          (v_buffer, v_buffer.stride(0), v_buffer.stride(1), v_buffer.stride(2), dv),
-                          partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale), split_cap=cap)
-    return ops.merge_stage2(partial, lse, o, None, splits, lens, batch, hq, hq, kv_len, S, split_cap=cap)
+        cap, S, plan = _plan_wide(lens, splits, S, batch, kv_len)
+    else:   # room in the workspaces for the splits the kernels may add (host arithmetic only)
+        cap, S, plan = MAX_SPLIT_TOKENS, ops.capped_splits(kv_len, S, MAX_SPLIT_TOKENS), None
+    partial, lse = ops.workspaces(batch, hq, S, dv, q.device)
+    ops.latent_stage1(q3, None, None,
+                      (k_buffer, k_buffer.stride(0), k_buffer.stride(1), k_buffer.stride(2), d), None,
+                      (v_buffer, v_buffer.stride(0), v_buffer.stride(1), v_buffer.stride(2), dv),
+                      partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale), split_cap=cap,
+                      split_plan=plan)
+    return ops.merge_stage2(partial, lse, o, None, splits, lens, batch, hq, hq, kv_len, S, split_cap=cap, split_plan=plan)
 
 
 def decode_attention_fwd_v_factorized(q, k_buffer, v_A_buffer, v_B_buffer, o, num_kv_splits, max_kv_splits,
@@ -79,24 +94,24 @@ def decode_attention_fwd_v_factorized(q, k_buffer, v_A_buffer, v_B_buffer, o, nu
     kv_len = k_buffer.shape[1]
     q3 = ops._q3(q)
     k_buffer, v_A_buffer = ops.as_rows(k_buffer), ops.as_rows(v_A_buffer)
-    wide = (hkv * d == 1024 and rv in (256, 384, 512)) or (hkv * d == 512 and rv == 512)
-    wide = wide and hq <= 32 and k_buffer.stride(2) == d
-    # one workgroup serves every head of a split in the wide form, so there are hkv times fewer workgroups than in the
-    # per-head form: its splits may be twice as long before the chip runs out of work
-    cap = MAX_SPLIT_TOKENS_WIDE if wide else 0
-    S = ops.capped_splits(kv_len, S, cap)
+    # 8 kv heads of 128 side by side in a token row: stage 1 serves every head of a split from one workgroup, and the value
+    # basis (shared by the heads) is read once per token instead of once per kv head
+    wide8 = hkv * d == 1024 and d == 128 and rv in (256, 384, 512) and hq <= 32 and k_buffer.stride(2) == d
+    # 512-wide token rows (4 x 128, 2 x 256 ...): the same form, with the block-diagonal query built here
+    wide4 = hkv * d == 512 and rv == 512 and hq <= 32 and k_buffer.stride(2) == d
+    cap, S, plan = _plan_wide(lens, splits, S, batch, kv_len) if (wide8 or wide4) else (0, S, None)
     partial, lse = ops.workspaces(batch, hq, S, rv, q.device)
-    if wide:
-        # all heads from one workgroup: the token's keys are one hkv*d-wide row against a block-diagonal query, and the
-        # value basis (shared by the heads) is read once per token instead of once per kv head
-        qbd = ops.blockdiag_q(q3, hkv)
-        ops.latent_stage1(qbd, None, None,
+    if wide4:
+        ops.latent_stage1(ops.blockdiag_q(q3, hkv), None, None,
                           (k_buffer, k_buffer.stride(0), k_buffer.stride(1), 0, hkv * d), None,
                           (v_A_buffer, v_A_buffer.stride(0), v_A_buffer.stride(1), 0, rv),
-                          partial, lse, None, splits, lens, batch, hq, 1, kv_len, S, float(sm_scale), split_cap=cap)
+                          partial, lse, None, splits, lens, batch, hq, 1, kv_len, S, float(sm_scale), split_cap=cap,
+                          split_plan=plan)
     else:
         ops.latent_stage1(q3, None, None,
                           (k_buffer, k_buffer.stride(0), k_buffer.stride(1), k_buffer.stride(2), d), None,
                           (v_A_buffer, v_A_buffer.stride(0), v_A_buffer.stride(1), 0, rv),
-                          partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale))
-    return ops.merge_stage2(partial, lse, o, v_B_buffer, splits, lens, batch, hq, hkv, kv_len, S, split_cap=cap)
+                          partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S, float(sm_scale), split_cap=cap,
+                          split_plan=plan)
+    return ops.merge_stage2(partial, lse, o, v_B_buffer, splits, lens, batch, hq, hkv, kv_len, S, split_cap=cap,
+                            split_plan=plan)

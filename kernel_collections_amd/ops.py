@@ -174,16 +174,17 @@ def blockdiag_q(q3: torch.Tensor, hkv: int) -> torch.Tensor:
 
 
 def latent_stage1(qn, qn_lo, qr, C, R, V, partial, lse, scores, num_kv_splits, kv_lens,
-                  batch, hq, groups, kv_len, max_splits, sm_scale, logit_cap=0.0, split_cap=0):
+                  batch, hq, groups, kv_len, max_splits, sm_scale, logit_cap=0.0, split_cap=0, split_plan=None):
     """C / R / V are `(tensor, stride_b, stride_l, stride_h, dim)` tuples or None.  `split_cap` > 0: no split longer than that
     many tokens (the kernels then scan sequence b with ``max(num_kv_splits[b], ceil(len_b / split_cap))`` splits; `max_splits`,
-    the split dimension of the workspaces, must cover ``ceil(kv_len / split_cap)``)."""
+    the split dimension of the workspaces, must cover ``ceil(kv_len / split_cap)``).  `split_plan`: the int32 device
+    array `plan_splits` returned; the cap in force is then the larger of the two and stage 1 takes its jobs from the list."""
     def op(x):
         return kv_operand(None) if x is None else kv_operand(*x)
     sd = dtype_code(scores.dtype) if scores is not None else 0
     check(_lib.lib().xkv_latent_stage1(
         q_operand(qn), ptr(qn_lo), q_operand(qr), op(C), op(R), op(V), ptr(partial), ptr(lse), ptr(scores), sd,
-        ptr(num_kv_splits), ptr(kv_lens), batch, hq, groups, kv_len, max_splits, int(split_cap),
+        ptr(num_kv_splits), ptr(kv_lens), batch, hq, groups, kv_len, max_splits, int(split_cap), ptr(split_plan),
         c_float(sm_scale), c_float(logit_cap), dtype_code(qn.dtype), stream_ptr(qn)), "xkv_latent_stage1")
 
 
@@ -206,7 +207,8 @@ def recon_stage1(q3, kA, kB, vA, partial, lse, scores, num_kv_splits, kv_lens, b
         "xkv_recon_stage1")
 
 
-def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, kv_len, max_splits, lse_out=None, split_cap=0):
+def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, kv_len, max_splits, lse_out=None, split_cap=0,
+                 split_plan=None):
     """out `[b,Hq,*]` (strides honoured on the first two axes).  `lse_out` `[b,Hq]` (any strides, fp32): log-sum-exp
     of the merged range.  Up-projections wider than 512 columns run as column blocks of 512."""
     dv = partial.shape[-1]
@@ -216,7 +218,7 @@ def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, 
     def call(o, w, d_out, sv, vdt, lo):
         check(_lib.lib().xkv_merge_stage2(
             ptr(partial), ptr(lse), ptr(o), ptr(w), c_int64(sv[0]), c_int64(sv[1]), c_int64(sv[2]), d_out, vdt,
-            ptr(num_kv_splits), ptr(kv_lens), batch, hq, hkv, kv_len, max_splits, int(split_cap), dv,
+            ptr(num_kv_splits), ptr(kv_lens), batch, hq, hkv, kv_len, max_splits, int(split_cap), ptr(split_plan), dv,
             c_int64(o.stride(0)), c_int64(o.stride(1)), dtype_code(o.dtype), ptr(lo), c_int64(sl[0]), c_int64(sl[1]),
             stream_ptr(partial)), "xkv_merge_stage2")
 
@@ -229,6 +231,17 @@ def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, 
         c1 = min(c0 + 512, vB.shape[-1])
         call(out[..., c0:c1], vB[..., c0:c1], c1 - c0, sv, vdt, lse_out if c0 == 0 else None)
     return out
+
+
+def plan_splits(kv_lens: torch.Tensor, num_kv_splits: torch.Tensor, max_splits: int, floor_tokens: int, target_jobs: int):
+    """The int32 device array `xkv_plan_splits` fills: [0] the smallest multiple of 32, not below `floor_tokens`, that cuts the
+    sequences of the batch into at most `target_jobs` splits; [1] the number of live (sequence, split) pairs; then the pairs.
+    Pass it as `split_plan` (with `split_cap=floor_tokens` and the same `max_splits`) to stage 1 and the merge."""
+    batch = kv_lens.numel()
+    plan = torch.empty(2 + 2 * batch * int(max_splits), dtype=torch.int32, device=kv_lens.device)
+    check(_lib.lib().xkv_plan_splits(ptr(kv_lens), ptr(num_kv_splits), batch, int(max_splits), int(floor_tokens),
+                                     int(target_jobs), ptr(plan), stream_ptr(kv_lens)), "xkv_plan_splits")
+    return plan
 
 
 def capped_splits(kv_len: int, max_kv_splits: int, cap_tokens: int) -> int:

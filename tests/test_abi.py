@@ -42,7 +42,7 @@ def test_argument_errors_are_reported_before_any_launch():
     ns = ctypes.c_void_p(16)
     # feature width 100 is outside the envelope (multiple of 32 required)
     rc = L.xkv_latent_stage1(q, null, _lib.QOperand(null, 0), kv, none, kv, ctypes.c_void_p(16), ctypes.c_void_p(16),
-                             null, 0, ns, null, 1, 4, 1, 8, 1, 0, 1.0, 0.0, _lib.XKV_BF16, null)
+                             null, 0, ns, null, 1, 4, 1, 8, 1, 0, null, 1.0, 0.0, _lib.XKV_BF16, null)
     assert rc == -2
     with pytest.raises(RuntimeError, match="envelope"):
         _lib.check(rc, "xkv_latent_stage1")
@@ -148,11 +148,15 @@ def test_split_cap_needs_room_in_the_workspace():
     kv = _lib.KVOperand(p16, 8192 * 128, 128, 0, 128)
     none = _lib.KVOperand(null, 0, 0, 0, 0)
     args = lambda max_splits, cap: (q, null, _lib.QOperand(null, 0), kv, none, kv, p16, p16, null, 0, p16, null,
-                                    1, 4, 1, 8192, max_splits, cap, 1.0, 0.0, _lib.XKV_BF16, null)
+                                    1, 4, 1, 8192, max_splits, cap, null, 1.0, 0.0, _lib.XKV_BF16, null)
     assert L.xkv_latent_stage1(*args(7, 1024)) == -1          # 8192 tokens at 1024 per split need 8 rows
     assert L.xkv_latent_stage1(*args(2, -5)) == -1
-    assert L.xkv_merge_stage2(p16, p16, p16, null, 0, 0, 0, 128, 0, p16, null, 1, 4, 1, 8192, 7, 1024, 128, 512, 128, _lib.XKV_BF16,
-                              null, 0, 0, null) == -1
+    assert L.xkv_merge_stage2(p16, p16, p16, null, 0, 0, 0, 128, 0, p16, null, 1, 4, 1, 8192, 7, 1024, null, 128, 512, 128,
+                              _lib.XKV_BF16, null, 0, 0, null) == -1
+    # a split plan's cap only raises the host's value, which is what bounds the workspaces: it needs one
+    dev_cap = lambda max_splits, cap: args(max_splits, cap)[:18] + (p16,) + args(max_splits, cap)[19:]
+    assert L.xkv_latent_stage1(*dev_cap(8, 0)) == -1
+    assert L.xkv_plan_splits(null, p16, 4, 8, 1024, 256, p16, null) == -1 and L.xkv_plan_splits(p16, p16, 4, 8, 0, 256, p16, null) == -1
     assert ops.capped_splits(8192, 2, 1024) == 8 and ops.capped_splits(8192, 16, 1024) == 16 and ops.capped_splits(8192, 2, 0) == 2
     assert ops.capped_splits(104212, 26, 1024) == 102
 

@@ -83,6 +83,36 @@ def test_ragged_4096_token_splits_with_long_sequences(dev, dtype, monkeypatch):
 
 
 # ------------------------------------------------------------------------------------ configuration 4, full size
+def test_split_plan_matches_brute_force(dev):
+    """xkv_plan_splits: the cap is the smallest multiple of 32, not below the floor, that cuts the batch into at most `jobs`
+    splits (against a linear search on the host), and the job list holds every live (sequence, split) pair exactly once,
+    whole splits before the last ones - for ragged batches, a batch larger than the job count, a floor that already
+    suffices, and callers that ask for more splits than the cap needs."""
+    import random
+    rnd = random.Random(5)
+    cases = [(config4_lengths(), 1024, 256), (config4_lengths(), 512, 64), ([5, 17, 33, 64], 32, 8),
+             ([4000] * 300, 1024, 256), ([100, 200, 300], 1024, 256)]
+    cases += [([rnd.randint(1, 200000) for _ in range(rnd.randint(1, 700))], 32 * rnd.randint(1, 64), rnd.randint(1, 512))
+              for _ in range(6)]
+    for k, (lens, floor, jobs) in enumerate(cases):
+        asked = [rnd.randint(1, 6) if k % 2 else 1 for _ in lens]
+        S = max(max(asked), -(-max(lens) // floor))
+        plan = ops.plan_splits(splits_t(lens, dev), splits_t(asked, dev), S, floor, jobs).cpu().tolist()
+        count = lambda cap: sum(-(-n // cap) for n in lens)
+        top = max(floor, -(-max(lens) // 32) * 32)
+        want = next((c for c in range(floor, top, 32) if count(c) <= jobs), top)
+        assert plan[0] == want, (len(lens), floor, jobs, plan[0], want)
+        live = []
+        for n, a in zip(lens, asked):
+            ns = max(a, -(-n // want))
+            per = -(-(-(-n // ns)) // 32) * 32
+            live.append(min(-(-n // per), S))
+        pairs = [(plan[2 + 2 * j], plan[3 + 2 * j]) for j in range(plan[1])]
+        assert plan[1] == sum(live) and sorted(pairs) == sorted((b, s) for b, l in enumerate(live) for s in range(l))
+        n_whole = sum(l - 1 for l in live)
+        assert all(s < live[b] - 1 for b, s in pairs[:n_whole]) and all(s == live[b] - 1 for b, s in pairs[n_whole:])
+
+
 @pytest.mark.parametrize("vfact", [False, True], ids=["plain", "v_factorised"])
 def test_config4_full_size(dev, vfact):
     """Target configuration 4 as configured: batch 32, lengths log-uniform in [1024, 131072], 32 q / 8 kv heads, d 128,
