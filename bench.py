@@ -31,8 +31,10 @@ PEAK_BF16_TFLOPS = 2500.0
 # HBM bytes of one stage-1 launch at the default c3 shape, from two rocprofv3 --pmc runs of this file
 # (FETCH_SIZE, WRITE_SIZE; each scaled by what the counter reads for --calib-copy's 512 MiB copies).
 # A counter cannot be read from inside the timed process, so the figure is recorded here.
-C3_STAGE1_HBM_BYTES = 535740 * 1024
-C5_RING_HBM_BYTES = 602896 * 1024     # same method, latent_ring_kernel at the default c5 shape
+C3_STAGE1_HBM_BYTES = 538148 * 1024     # recon_fast_kernel 2 x 267013.5 + 2056.1 KiB, pack_b_kernel 2 x 520.5 + 1024 KiB
+C5_RING_HBM_BYTES = 604800 * 1024       # same method, latent_ring_kernel at the default c5 shape (2 x 298272.1 + 8256.0 KiB)
+C2_RING_HBM_BYTES = 151785 * 1024       # latent_ring_kernel, scores mode, default c2 shape (2 x 67700.4 + 16384.0 KiB)
+C4_RING_HBM_BYTES = 3022744 * 1024      # latent_ring_kernel at c4 plain with the planned split length (2 x 1509401.8 + 3940.0 KiB)
 OUT_ATOL, SCORE_RTOL = 2e-2, 1e-2     # the parity bars (attention output max-abs, scores max|delta| / max|ref|)
 
 
@@ -379,7 +381,7 @@ def bench_c2(args, dev):
         "config": {"workload": "c2 qAB_no_pe scores: batch 8, 32q/8kv, d128, L16384, rank 512, bf16 in / fp32 out", "kv_splits": S,
                    "buffers_rotated": nbuf},
         "roofline": {"bound": "hbm", "kernel": "latent_ring_kernel(scores)", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None if args.splits else C2_RING_HBM_BYTES,
                      "kernel_avg_us": round(k_avg_ms * 1e3, 2), "kernel_median_us": round(k_med_ms * 1e3, 2),
                      "kernel_avg_us_one_buffer": round(warm_avg_ms * 1e3, 2), "algorithmic_bytes": algo_bytes},
         "parity_vs_oracle": parity,
@@ -512,9 +514,10 @@ def bench_c4(args, dev, vfact):
                    "kv_splits_max_in_the_kernel": max(max(s_, -(-n // limit)) for n, s_ in zip(lens, ns_l)),
                    "workgroups_with_work": sum(max(s_, -(-n // limit)) for n, s_ in zip(lens, ns_l)),
                    "compute_units": ops.num_cus()},
-        "roofline": {"bound": "hbm", "kernel": "latent_ring_kernel" if vfact else "latent_stage1_kernel",
+        "roofline": {"bound": "hbm", "kernel": "latent_ring_kernel",
                      "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
+                     "traffic": C4_RING_HBM_BYTES if (not vfact and split == 4096) else None,
                      "note": "whole call (stage 1 + merge) over algorithmic bytes", "algorithmic_bytes": algo_bytes},
         "caller_splits_as_they_are_us": round(asis_ms * 1e3 / args.steps, 2),
         "parity_vs_oracle": parity,

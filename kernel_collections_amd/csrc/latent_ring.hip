@@ -58,12 +58,6 @@ __device__ __forceinline__ f32x4 mfma16k16(_Float16, s16x4r a, s16x4r b, f32x4 c
   return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4r, a), __builtin_bit_cast(f16x4r, b), c, 0, 0, 0);
 }
 
-#ifdef XKV_RING_STAMPS
-__device__ unsigned long long ring_stamps[4096 * 8];
-#define STAMP(i) do { if (lane == 0) ring_stamps[(blockIdx.x & 4095) * 8 + (i)] = wall_clock64(); } while (0)
-#else
-#define STAMP(i)
-#endif
 constexpr int RING_QD = 2;      // tiles per loader wave in flight in registers (deeper queues only lengthen the start); >= 2
 enum { RING_SCORES = 0, RING_VSHARED = 1, RING_VDISTINCT = 2, RING_VHEADS = 3 };
 constexpr int RING_DVH = 128;   // head width of the per-head value rows (RING_VHEADS)
@@ -134,7 +128,6 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
   const int tb = wave % NTB, kh = wave / NTB;
   const int iw = wave - 4;                        // index among the loader waves (negative: a compute wave)
 
-  if (wave == 0) STAMP(0);
   const int wg = xcd_cluster_remap(blockIdx.x, p.groups);   // the kv groups of one (sequence, split) share an L2
   if (wg >= p.total_wg) return;
   const int group = wg % p.groups;
@@ -153,7 +146,6 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
   const int hg = p.hq / p.groups, h0 = group * hg;
   const int ntiles = (end - start + TN - 1) / TN;
   const int last = end - 1;
-  if (wave == 0) STAMP(1);
 
   // ---- LDS carve-up -------------------------------------------------------------------------------------------
   unsigned char* ring = smem;
@@ -224,7 +216,6 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
     // next iteration needs it.  Every queue entry is loaded at one place in the code and stored at one place: the loads
     // are invisible to the compiler, and a register copy between two such places would read a value that has not landed.
     // Tiles past the end are fetched too (clamped rows, never used): the vmcnt arithmetic counts on QD - 1 younger tiles.
-    if (wave == 4) STAMP(2);
     for (int j0 = 0; j0 <= ntiles + QD; j0 += QD) {   // j0 stays a multiple of QD, so the queue index below is static
 #pragma unroll
       for (int u = 0; u < QD; ++u) {
@@ -234,7 +225,6 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
           if (k >= 0) hand_on(k, rq[u]);
           fetch(j, rq[u]);
           if (j == 0) {
-            if (wave == 4) STAMP(5);
             __syncthreads();                           // start: the compute waves hold their query loads back until here
           }
           if (j == 1 && S::qst(LO)) __syncthreads();   // the compute waves' barrier between staging the query rows and reading them
@@ -352,7 +342,6 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
       if (LO) asm volatile("" : "+v"(qlo[k][hb]));
     }
 
-  if (wave == 0) STAMP(3);
   // ---- running state ---------------------------------------------------------------------------------------------
   const int srow = tid / TPH, ssub = tid % TPH;
   float m_run = NEG_INF, l_run = 0.f;
@@ -366,7 +355,6 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
 
   for (int t = 0; t < ntiles; ++t) {
     __syncthreads();                  // A: tile t is in its slot; every wave is past PV / score write of tile t-1
-    if (wave == 0 && t == 0) STAMP(4);
     const unsigned char* slot = ring + (t % RSLOT) * SLOT;
     const int base = start + t * TN;
 
@@ -507,7 +495,6 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
       }
     }
   }
-  if (wave == 0) STAMP(6);
   if (SCORES) return;
 
   // ---- epilogue: normalise, write partial + lse --------------------------------------------------------------------
@@ -639,9 +626,3 @@ int launch_ring(const RingParams& p, int batch, bool vshared, int dtype, hipStre
 }
 
 }  // namespace xkv
-
-#ifdef XKV_RING_STAMPS
-extern "C" int xkv_debug_stamps(unsigned long long* host, int n) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(xkv::ring_stamps), sizeof(unsigned long long) * n);
-}
-#endif
