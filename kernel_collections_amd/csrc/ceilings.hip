@@ -124,7 +124,8 @@ static int launch_stream(const void* src, int64_t bytes, int wgs, float* out, hi
   const size_t shm = TO_LDS ? (size_t)4 * DEPTH * 8192 : 0;
   auto kern = ceiling_stream_kernel<TO_LDS, DEPTH>;
   if (TO_LDS) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
+    static DynLds lds;
+    hipError_t e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), (int)shm);
     if (e != hipSuccess) return (int)e;
   }
   kern<<<dim3(wgs), dim3(256), shm, st>>>(reinterpret_cast<const unsigned char*>(src), steps, out);

@@ -335,8 +335,8 @@ static int launch_latent(const LatentParams& p, int batch, hipStream_t st) {
   shm += (size_t)HB * (TN + 4) * 4 + (size_t)HB * (TN + 8) * 2 + HB * 4 + HB * 8;
   if (shm > 160 * 1024) return XKV_EUNSUPPORTED;
   auto kern = latent_stage1_kernel<T, NHB, TN, NVB_MAX, NPK_C, NPK_R, NPK_V, VSHARED, SCORES_ONLY>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)shm);
+  static DynLds lds;
+  hipError_t e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), (int)shm);
   if (e != hipSuccess) return (int)e;
   const int total = batch * p.groups * p.max_splits;
   const int grid = xcd_grid(total, p.groups);

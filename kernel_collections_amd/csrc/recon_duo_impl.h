@@ -467,7 +467,8 @@ int launch_duo_t(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, 
   const int nb = sBb == 0 ? 1 : batch;   // one packed copy when the factor is shared by the batch
   duo_pack_b_kernel<T, RK><<<dim3(p.hkv, nb, 16), dim3(256), 0, st>>>((const T*)kB, (T*)p.Bp, sBb, sBh, sBr, p.hkv);
   auto kern = recon_duo_kernel<T, RK, RV, MODE>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, S::SHM);
+  static DynLds lds;
+  hipError_t e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), S::SHM);
   if (e != hipSuccess) return (int)e;
   const int total = batch * p.hkv * p.max_splits;
   kern<<<dim3(xcd_grid(total, p.hkv)), dim3(64 * NW), S::SHM, st>>>(p);

@@ -504,8 +504,8 @@ int launch_recon_fast_t(const FastParams& p, const void* kB, int64_t sBb, int64_
   const int nb = sBb == 0 ? 1 : batch;   // one packed copy when the factor is shared by the batch
   pack_b_kernel<T><<<dim3(p.hkv, nb, 32), dim3(256), 0, st>>>((const T*)kB, (T*)p.Bp, sBb, sBh, sBr, p.hkv);
   auto kern = p.scores ? recon_fast_kernel<T, true> : recon_fast_kernel<T, false>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)FAST_SHM);
+  static DynLds lds[2];
+  hipError_t e = ensure_dynamic_lds(lds[p.scores ? 1 : 0], reinterpret_cast<const void*>(kern), (int)FAST_SHM);
   if (e != hipSuccess) return (int)e;
   const int total = batch * p.hkv * p.max_splits;
   kern<<<dim3(xcd_grid(total, p.hkv)), dim3(256), FAST_SHM, st>>>(p);

@@ -329,8 +329,8 @@ static int launch_recon(const ReconParams& p, int batch, hipStream_t st) {
   if (!VSHARED && !SCORES_ONLY) shm += (size_t)RTN * ldv * 2;
   shm += 4 * 16 * (RTN + 4) * 4 + 16 * (RTN + 8) * 2 + 16 * 4 + 16 * 8;
   auto kern = recon_stage1_kernel<T, NKS, EXACT, NVB_MAX, VSHARED, SCORES_ONLY>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)shm);
+  static DynLds lds;
+  hipError_t e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), (int)shm);
   if (e != hipSuccess) return (int)e;
   const int total = batch * p.hkv * p.max_splits;
   kern<<<dim3(xcd_grid(total, p.hkv)), dim3(256), shm, st>>>(p);

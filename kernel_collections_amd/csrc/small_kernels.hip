@@ -376,8 +376,8 @@ static int launch_merge(const float* partial, const float* lse, void* out, const
   return launch_status();
 }
 
-// plan[0]: smallest multiple of 32 >= floor_tokens with sum_b ceil(len_b / cap) <= target_jobs, by bisection over cap / 32
-// (the job count falls monotonically as the cap grows).  Then the job list: sequence b has n_b = effective_splits(len_b,
+// plan[0]: smallest multiple of 32 >= floor_tokens with sum_b ceil(len_b / cap) <= target_jobs, by a 256-ary search over
+// cap / 32 (the job count falls monotonically as the cap grows).  Then the job list: sequence b has n_b = effective_splits(len_b,
 // num_splits[b], cap) splits of which the live ones are a prefix; whole splits first (sequence-major), every sequence's last
 // live split - the short one - after them.  One workgroup; thread t handles sequences t, t + 256, ...
 __global__ __launch_bounds__(256) void plan_splits_kernel(const int32_t* __restrict__ kv_lens, const int32_t* __restrict__ num_splits,
@@ -405,12 +405,35 @@ __global__ __launch_bounds__(256) void plan_splits_kernel(const int32_t* __restr
   lm = block_reduce(lm, true);
   int lo = cdiv(floor_tokens > 32 ? floor_tokens : 32, 32), hi = cdiv(lm > 32 ? lm : 32, 32);   // in units of 32 tokens
   if (hi < lo) hi = lo;
-  while (lo < hi) {   // if even one job per sequence is too many, this ends on the longest length
-    const int mid = (lo + hi) >> 1, cap = mid * 32;
-    int jobs = 0;
-    for (int b = threadIdx.x; b < batch; b += 256) jobs += cdiv(kv_lens[b] > 0 ? kv_lens[b] : 0, cap);
-    jobs = block_reduce(jobs, false);
-    if (jobs <= target_jobs) hi = mid; else lo = mid + 1;
+  // 256-ary search over [lo, hi]: the range is cut into 256 blocks and thread t tests the LAST cap of block t; the answer
+  // lies in the first block whose last cap fits.  If nothing fits - even one job per sequence is too many - it is hi, the
+  // longest length.
+  __shared__ int first_fit[4];
+  while (lo < hi) {
+    const int stride = cdiv(hi - lo + 1, 256);
+    const int blk_lo = lo + threadIdx.x * stride;
+    int blk_hi = blk_lo + stride - 1;
+    blk_hi = blk_hi < hi ? blk_hi : hi;
+    bool fits = false;
+    if (blk_lo <= hi) {
+      const int cap = blk_hi * 32;
+      int jobs = 0;
+      for (int b = 0; b < batch; ++b) jobs += cdiv(kv_lens[b] > 0 ? kv_lens[b] : 0, cap);
+      fits = jobs <= target_jobs;
+    }
+    const unsigned long long m = __builtin_amdgcn_ballot_w64(fits);
+    __syncthreads();            // first_fit is free again
+    if (lane == 0) first_fit[wave] = m ? wave * 64 + (int)__builtin_ctzll(m) : 1 << 30;
+    __syncthreads();
+    int t = first_fit[0];
+#pragma unroll
+    for (int i = 1; i < 4; ++i) t = first_fit[i] < t ? first_fit[i] : t;
+    if (t == 1 << 30) { lo = hi; break; }
+    const int new_lo = lo + t * stride;
+    int new_hi = new_lo + stride - 1;
+    new_hi = new_hi < hi ? new_hi : hi;
+    lo = new_lo;
+    hi = new_hi;                // fits; with stride 1 this ends the search
   }
   const int cap = lo * 32;
   // live splits of a sequence, in the arithmetic of split_bounds

@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 
 #include "../../include/xkv_hip.h"
 
@@ -130,6 +131,22 @@ __device__ __forceinline__ int xcd_cluster_remap(int id, int cluster) {
   return ((j / cluster) * 8 + xcd) * cluster + (j % cluster);
 }
 inline int xcd_grid(int total_wg, int cluster) { return ((total_wg / cluster + 7) & ~7) * cluster; }
+
+// hipFuncSetAttribute costs host microseconds on every call: a launcher asks for a kernel's dynamic LDS size once per device
+// (again only if a later call needs more).  One DynLds per kernel instantiation, as a function-local static.
+struct DynLds {
+  std::atomic<int> bytes[16];
+  DynLds() { for (auto& b : bytes) b.store(0, std::memory_order_relaxed); }
+};
+inline hipError_t ensure_dynamic_lds(DynLds& st, const void* kernel, int bytes) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev >= 0 && dev < 16 && st.bytes[dev].load(std::memory_order_acquire) >= bytes) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && dev >= 0 && dev < 16) st.bytes[dev].store(bytes, std::memory_order_release);
+  return e;
+}
 
 inline int launch_status() {
   hipError_t e = hipGetLastError();
