@@ -183,12 +183,21 @@ def test_plain_vonly_konly_mla_consistency():
 
 
 def test_softmax_cast_order():
-    # probabilities are formed in fp32 and cast to the query dtype BEFORE the value product
-    q = rnd(1, 2, 1, 8).to(torch.bfloat16)
-    kA, kB = rnd(1, 20, 4, seed=2).to(torch.bfloat16), rnd(1, 1, 4, 8, seed=3).to(torch.bfloat16)
-    out = oracle.gqa_factorized(q, kA, kB, kA, kB)
+    """Probabilities are formed in fp32 and rounded to the query dtype BEFORE the value product (attention.py:330).  The two
+    orders give different results in bf16, and the oracle equals the rounded-first one bit for bit."""
+    b, hq, hkv, d, L = 1, 4, 2, 16, 64
+    q, K, V = (rnd(b, hq, d, seed=1).to(torch.bfloat16), rnd(b, L, hkv, d, seed=2).to(torch.bfloat16),
+               rnd(b, L, hkv, d, seed=3).to(torch.bfloat16))
+    out = oracle.gqa_plain(q, K, V, 0.7)
     assert out.dtype == torch.bfloat16
     assert oracle.softmax_pv(torch.zeros(1, 4), torch.bfloat16).dtype == torch.bfloat16
+    g = hq // hkv
+    s = torch.matmul(q.reshape(b, hkv, g, d), K.transpose(1, 2).transpose(-1, -2)) * 0.7
+    p32 = torch.softmax(s, dim=-1, dtype=torch.float32)
+    rounded_first = torch.matmul(p32.to(torch.bfloat16), V.transpose(1, 2)).reshape(b, hq, d)
+    rounded_last = torch.matmul(p32, V.transpose(1, 2).float()).to(torch.bfloat16).reshape(b, hq, d)
+    assert torch.equal(out, rounded_first)
+    assert not torch.equal(rounded_first, rounded_last), "the cast order must be observable for this test to pin anything"
 
 
 # ----------------------------------------------------------------------------- split-K + merge
