@@ -81,7 +81,8 @@ struct RingShape {
   // it fits beside the ring
   static constexpr int QSTRIDE = (DN + (HAS_R ? 64 : 0)) * 2 + 16;
   static constexpr int qst_bytes(bool lo) { return HB * QSTRIDE * (lo ? 2 : 1); }
-  static constexpr bool qst(bool lo) { return SHM + qst_bytes(lo) <= 160 * 1024; }
+  // (not for the 1024-wide form: its query arrives as compact 128-wide rows and is expanded in registers)
+  static constexpr bool qst(bool lo) { return DN != 1024 && SHM + qst_bytes(lo) <= 160 * 1024; }
   static constexpr int shm(bool lo) { return SHM + (qst(lo) ? qst_bytes(lo) : 0); }
   static_assert(SHM <= 160 * 1024, "ring does not fit the LDS");
 };
