@@ -126,6 +126,11 @@ typedef struct {
  * Dead splits write nothing.  partial is [batch, hq, max_splits, V.dim] fp32, lse [batch, hq, max_splits] fp32.
  * Envelope: heads per kv group <= 32; C.dim % 32 == 0, <= 1024; R.dim % 32 == 0, <= 128;
  *           V.dim % 64 == 0, <= 512.
+ * Plain keys of 8 kv heads x 128 stored side by side in a token row (n_kv_groups == 8, C.dim == 128, C.stride_h == 128,
+ * hq <= 32), with values laid out the same way or as one shared 256 / 384 / 512-wide row (V.stride_h == 0), are served
+ * by one workgroup per (sequence, split) for ALL heads: the token's keys are then one 1024-wide row against a block-
+ * diagonal query that the kernel builds from qn.  Same call, same result; only the work distribution differs (one job
+ * per split instead of eight), which is what xkv_plan_splits' target_jobs should count.
  * Replaces _fwd_grouped_kernel_stage1[grid] at flash_decoding/gqa.py:205-237,
  * flash_decoding/mla.py (same launcher, :243-283), flash_decoding/mla2/stage1.py:213-249,
  * flash_recontruction/fused_attention/no_pe/v1.py:227-262 (and v2.py / v1_k_only.py twins) and,

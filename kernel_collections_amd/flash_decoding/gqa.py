@@ -6,7 +6,9 @@ Call surface of the reference's flash_decoding/gqa.py:339-434 (``decode_attentio
   * ``decode_attention_fwd_v_factorized``: K plain, ``V = v_A @ v_B`` (the eager semantics of
     ``group_query_attention_factorized_v_only``, reference attention.py:202-274) as a split-K kernel
     that accumulates ``P @ v_A`` in rank space and multiplies by ``v_B`` after the merge.
-Split ranges follow gqa.py:95-99 exactly; ``sm_scale`` multiplies the scores (gqa.py:122).
+Split ranges follow gqa.py:95-99 exactly; ``sm_scale`` multiplies the scores (gqa.py:122).  The caller's split counts are a
+lower bound: a sequence is cut into more splits when that is what fills the device (split-K is exact under the merge), by a
+fixed cap in the per-head form and by a per-call plan computed on the device in the all-heads forms.
 """
 from __future__ import annotations
 
