@@ -113,6 +113,33 @@ def test_split_plan_matches_brute_force(dev):
         assert all(s < live[b] - 1 for b, s in pairs[:n_whole]) and all(s == live[b] - 1 for b, s in pairs[n_whole:])
 
 
+@pytest.mark.parametrize("hkv,d", [(4, 128), (2, 64)], ids=["ring_not_eligible_4x128", "2x64"])
+def test_split_plan_with_the_per_head_kernels(dev, hkv, d):
+    """A split plan passed straight to xkv_latent_stage1 / xkv_merge_stage2 for head layouts the all-heads form does not
+    serve (the register-staged kernel takes its jobs from the list too): same attention as without a plan."""
+    b, hq, scale = 5, 8, d ** -0.5
+    lens = [3000, 70, 1025, 2048, 333]
+    L = max(lens)
+    q, K, V = randn_dev((b, hq, d), 1.0, dev, BF, 1), randn_dev((b, L, hkv, d), 1.0, dev, BF, 2), randn_dev((b, L, hkv, d), 1.0, dev, BF, 3)
+    ref = oracle.ragged_apply(oracle.gqa_plain, lens, f32(q.cpu(), K.cpu(), V.cpu()), (None, 1, 1), sm_scale=scale)
+    kl, ns = splits_t(lens, dev), splits_t([1] * b, dev)
+    floor = 256
+    S = ops.capped_splits(L, 1, floor)
+    outs = []
+    for jobs in (12, 4, None):     # a plan that lengthens the splits, one that ends on one job per sequence, no plan
+        plan = None if jobs is None else ops.plan_splits(kl, ns, S, floor, jobs)
+        partial, lse = ops.workspaces(b, hq, S, d, dev)
+        partial.fill_(float("nan"))
+        ops.latent_stage1(q, None, None, (K, K.stride(0), K.stride(1), K.stride(2), d), None,
+                          (V, V.stride(0), V.stride(1), V.stride(2), d), partial, lse, None, ns, kl, b, hq, hkv, L, S, scale,
+                          split_cap=floor, split_plan=plan)
+        o = torch.empty_like(q)
+        ops.merge_stage2(partial, lse, o, None, ns, kl, b, hq, hq, L, S, split_cap=floor, split_plan=plan)
+        check_out(o, ref, f"per-head kernels, plan for {jobs} jobs")
+        outs.append(o)
+    assert max_abs(outs[0], outs[2]) < 4e-3 and max_abs(outs[1], outs[2]) < 4e-3
+
+
 @pytest.mark.parametrize("vfact", [False, True], ids=["plain", "v_factorised"])
 def test_config4_full_size(dev, vfact):
     """Target configuration 4 as configured: batch 32, lengths log-uniform in [1024, 131072], 32 q / 8 kv heads, d 128,
