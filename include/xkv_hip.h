@@ -143,6 +143,20 @@ int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_operand qr,
                       int batch, int hq, int n_kv_groups, int kv_len, int max_splits, int split_cap_tokens,
                       const int32_t* split_plan, float sm_scale, float logit_cap, int dtype, void* stream);
 
+/* Split-K stage 1 over scores that already exist: per live split, the online softmax of scores[b, h, start:end] and
+ *   partial[b,h,i,:] = sum_l exp(s - m) V[b,l,:] / den ;  lse[b,h,i] = m + log(den)
+ * with scores fp32 [batch, hq, kv_len] as written (scaled) by the scores_out mode of xkv_recon_stage1 or
+ * xkv_latent_stage1, and V one row per token shared by every head (V.stride_h == 0; V.dim 256 / 384 / 512).  It is the
+ * second pass of a fused decode whose value basis differs from its key basis: the first pass rebuilds and rotates the keys
+ * at the rate of the scores-only kernel, this one streams v_A once for all heads.  Splits, kv_lens, split_cap_tokens and
+ * split_plan as in xkv_latent_stage1; the softmax weights are rounded to `dtype` before P.V as everywhere else.
+ * hq <= 32; kv_len % 4 == 0.  No single reference launch: the reference fuses this into its stage-1 kernels
+ * (fused_attention/no_pe/v1.py:40-190) and has no RoPE-aware fused decode at all. */
+int xkv_softmax_pv_stage1(const float* scores, xkv_kv_operand V, float* partial, float* lse,
+                          const int32_t* num_kv_splits, const int32_t* kv_lens,
+                          int batch, int hq, int kv_len, int max_splits, int split_cap_tokens, const int32_t* split_plan,
+                          int dtype, void* stream);
+
 /* Split-K stage 1 with fused key reconstruction and RoPE:
  *
  *   K[b,kh,l,:]  = kA[b,l,:] @ kB[b,kh,:,:]                      (rank x 128, fp32 accumulate)

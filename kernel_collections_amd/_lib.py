@@ -17,7 +17,7 @@ ABI_VERSION = 5
 EXPORTS = (
     "xkv_abi_version", "xkv_error_string", "xkv_rope_table", "xkv_absorb_q",
     "xkv_blockdiag_q", "xkv_latent_stage1", "xkv_recon_stage1", "xkv_recon_workspace_bytes", "xkv_merge_stage2",
-    "xkv_recon_stage1_static", "xkv_rope_apply", "xkv_ceiling_mfma", "xkv_ceiling_stream", "xkv_plan_splits",
+    "xkv_recon_stage1_static", "xkv_rope_apply", "xkv_ceiling_mfma", "xkv_ceiling_stream", "xkv_plan_splits", "xkv_softmax_pv_stage1",
 )
 STATIC_SCRATCH_BYTES = 4 << 20
 XKV_ESCRATCH = -5
@@ -71,6 +71,9 @@ def _declare(lib):
     lib.xkv_merge_stage2.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int,
                                      c_int64, c_int64, c_int, c_void_p, c_int64, c_int64, c_void_p]
+    lib.xkv_softmax_pv_stage1.restype = c_int
+    lib.xkv_softmax_pv_stage1.argtypes = [c_void_p, KVOperand, c_void_p, c_void_p, c_void_p, c_void_p,
+                                          c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p]
     lib.xkv_plan_splits.restype = c_int
     lib.xkv_plan_splits.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]
 

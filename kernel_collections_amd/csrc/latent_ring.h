@@ -26,5 +26,8 @@ typedef LatentParams RingParams;
 // absorbed key basis or under plain per-head keys taken as one 1024-wide row.  Everything else runs the register-staged kernel.
 bool ring_eligible(const RingParams& p, bool vshared);
 int launch_ring(const RingParams& p, int batch, bool vshared, int dtype, hipStream_t st);
+// Softmax + P.V over scores that are an input (p.scores: fp32 [batch, hq, kv_len], already scaled); p.C = the value rows
+// (256 / 384 / 512 wide, one row per token for every head), p.groups == 1, hq <= 32, kv_len % 4 == 0.
+int launch_ring_given(const RingParams& p, int batch, int dtype, hipStream_t st);
 
 }  // namespace xkv

@@ -59,7 +59,7 @@ __device__ __forceinline__ f32x4 mfma16k16(_Float16, s16x4r a, s16x4r b, f32x4 c
 }
 
 constexpr int RING_QD = 2;      // tiles per loader wave in flight in registers (deeper queues only lengthen the start); >= 2
-enum { RING_SCORES = 0, RING_VSHARED = 1, RING_VDISTINCT = 2, RING_VHEADS = 3 };
+enum { RING_SCORES = 0, RING_VSHARED = 1, RING_VDISTINCT = 2, RING_VHEADS = 3, RING_VGIVEN = 4 };
 constexpr int RING_DVH = 128;   // head width of the per-head value rows (RING_VHEADS)
 
 template <int TN, int DN, bool HAS_R, int VMODE, int NHB, int DVW>
@@ -69,7 +69,7 @@ struct RingShape {
   static constexpr int CBYTES = TN * CROW;
   static constexpr int RBYTES = HAS_R ? TN * 128 : 0;
   static constexpr int VROW = DVW * 2 + 16;                // padded V row (distinct-V mode)
-  static constexpr int VBYTES = VMODE >= RING_VDISTINCT ? TN * VROW : 0;
+  static constexpr int VBYTES = (VMODE == RING_VDISTINCT || VMODE == RING_VHEADS) ? TN * VROW : 0;
   static constexpr int SLOT = CBYTES + RBYTES + VBYTES;
   static constexpr int KSPLIT = 4 / (TN / 16);             // k-ranges (waves per 16-token block)
   static constexpr int SP = TN + 4;                        // partial-score row stride (floats)
@@ -82,7 +82,7 @@ struct RingShape {
   static constexpr int QSTRIDE = (DN + (HAS_R ? 64 : 0)) * 2 + 16;
   static constexpr int qst_bytes(bool lo) { return HB * QSTRIDE * (lo ? 2 : 1); }
   // (not for the 1024-wide form: its query arrives as compact 128-wide rows and is expanded in registers)
-  static constexpr bool qst(bool lo) { return DN != 1024 && SHM + qst_bytes(lo) <= 160 * 1024; }
+  static constexpr bool qst(bool lo) { return DN != 1024 && VMODE != RING_VGIVEN && SHM + qst_bytes(lo) <= 160 * 1024; }
   static constexpr int shm(bool lo) { return SHM + (qst(lo) ? qst_bytes(lo) : 0); }
   static_assert(SHM <= 160 * 1024, "ring does not fit the LDS");
 };
@@ -92,13 +92,17 @@ struct RingShape {
 // DN features of the C row / V is a second, DVW-wide row stream / V is a second stream of DVW / 128 per-kv-head value
 // rows of 128 features (plain values under absorbed factorised keys): the workgroup serves every query head, wave w
 // accumulates kv heads 2w, 2w+1, and query head h multiplies the values of kv head h / (heads per kv head).
+// RING_VGIVEN: no query at all - the scaled scores [b, hq, kv_len] (fp32) are an input, the C rows are the values: softmax
+// and P.V over a value basis of its own, behind a kernel that produced the scores (two-pass fused decode).
 // DN 1024 means eight plain kv heads of 128 side by side in a token row, against compact query rows [b, hq, 128].
 template <typename T, int TN, int NHB, bool LO, int DN, bool HAS_R, int VMODE, int DVW>
 __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
   static_assert(DN != 1024 || (!LO && !HAS_R), "the 1024-wide form is plain per-head keys");
   typedef typename Elem<T>::vec8 vec8;
   typedef RingShape<TN, DN, HAS_R, VMODE, NHB, DVW> S;
-  constexpr bool SCORES = VMODE == RING_SCORES, V2 = VMODE >= RING_VDISTINCT, VHEADS = VMODE == RING_VHEADS;
+  constexpr bool SCORES = VMODE == RING_SCORES, V2 = VMODE == RING_VDISTINCT || VMODE == RING_VHEADS, VHEADS = VMODE == RING_VHEADS;
+  constexpr bool GIVEN = VMODE == RING_VGIVEN;
+  static_assert(!GIVEN || (!LO && !HAS_R && TN == 32), "given scores: plain 32-token tiles of value rows");
   constexpr int VIPR = DVW > 512 ? DVW / 512 : 1;   // load instructions per V row
   constexpr int KVH = DVW / RING_DVH, KVW = VHEADS ? KVH / 4 : 1;   // kv heads of a value row, per wave
   constexpr int HB = S::HB, CROW = S::CROW, CBYTES = S::CBYTES, VROW = S::VROW, SLOT = S::SLOT, RSLOT = S::RSLOT;
@@ -115,7 +119,7 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
   constexpr int RPW = TN / 4;                     // rows per loader wave per tile
   constexpr int LPT = RPW * IPR + (HAS_R ? 1 : 0) + (V2 ? RPW * VIPR : 0);   // loads per loader wave per tile
   static_assert((QD - 1) * LPT <= 63, "vmcnt holds 6 bits");
-  constexpr int DV = VMODE == RING_VSHARED ? DN : VHEADS ? RING_DVH : DVW;   // value features of an output row
+  constexpr int DV = (VMODE == RING_VSHARED || GIVEN) ? DN : VHEADS ? RING_DVH : DVW;   // value features of an output row
   constexpr int NVB = VHEADS ? RING_DVH / 16 : DV / 64;   // 16-feature blocks per wave (per kv head under VHEADS)
   constexpr int NA2 = VHEADS ? KVW : NHB;
   static_assert(!VHEADS || (TN == 16 && KVH % 4 == 0), "per-head values: 16-token tiles, kv heads split over 4 waves");
@@ -245,7 +249,9 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
   // ---- query operands in registers: lane (n16 = head row, g4) holds q[head][32 ks + 8 g4 .. +8] for its k-range ----
   vec8 qreg[KS_W][NHB], qlo[LO ? KS_W : 1][NHB];
   const int ks0 = kh * KS_W;
-  if constexpr (S::qst(LO)) {
+  if constexpr (GIVEN) {
+    // no query operands
+  } else if constexpr (S::qst(LO)) {
     // Whole rows, coalesced, each read once per workgroup, into the LDS; every lane then picks its operand pieces from there.
     // (Read straight into the operand layout, a load instruction touches 16 half-used cache lines and two waves fetch
     // the same rows: several microseconds at the start of a kernel that lasts tens.)
@@ -335,13 +341,26 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
     }
   }
   // Wait for the query loads here, once, rather than at their first uses inside the loop.
+  if constexpr (!GIVEN) {
 #pragma unroll
-  for (int k = 0; k < KS_W; ++k)
+    for (int k = 0; k < KS_W; ++k)
 #pragma unroll
-    for (int hb = 0; hb < NHB; ++hb) {
-      asm volatile("" : "+v"(qreg[k][hb]));
-      if (LO) asm volatile("" : "+v"(qlo[k][hb]));
-    }
+      for (int hb = 0; hb < NHB; ++hb) {
+        asm volatile("" : "+v"(qreg[k][hb]));
+        if (LO) asm volatile("" : "+v"(qlo[k][hb]));
+      }
+  }
+  // Given scores: thread -> 4 tokens of one head row of the tile (8 threads per row), fetched one tile ahead into registers.
+  const int gv_row = tid >> 3, gv_c0 = (tid & 7) * 4;
+  const bool gv_active = GIVEN && gv_row < HB;
+  auto given_tile = [&](int t) -> f32x4 {
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    const int tok = start + t * TN + gv_c0;
+    if (gv_active && gv_row < hg && t < ntiles && tok + 4 <= p.kv_len)    // kv_len % 4 == 0: whole 16-byte pieces or nothing
+      v = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.scores) + ((int64_t)b * p.hq + h0 + gv_row) * p.kv_len + tok);
+    return v;
+  };
+  f32x4 gv_next = given_tile(0);
 
   // ---- running state ---------------------------------------------------------------------------------------------
   const int srow = tid / TPH, ssub = tid % TPH;
@@ -360,7 +379,10 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
     const int base = start + t * TN;
 
     // ---- QK: partial scores of token block tb over this wave's k-range -------------------------------------------
-    {
+    if constexpr (GIVEN) {               // the scores are an input: this tile's into the first partial plane, the next tile's on their way
+      if (gv_active) *reinterpret_cast<f32x4*>(s_part + gv_row * SP + gv_c0) = gv_next;
+      gv_next = given_tile(t + 1);
+    } else {
       f32x4 sacc[NHB];
 #pragma unroll
       for (int hb = 0; hb < NHB; ++hb) sacc[hb] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -425,7 +447,7 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
         const int c = ssub * TPT + i;
         float s = 0.f;
 #pragma unroll
-        for (int kr = 0; kr < KSPLIT; ++kr) s += s_part[(kr * HB + srow) * SP + c];
+        for (int kr = 0; kr < (GIVEN ? 1 : KSPLIT); ++kr) s += s_part[(kr * HB + srow) * SP + c];
         s *= p.sm_scale;
         if (p.logit_cap > 0.f) s = p.logit_cap * tanhf(s / p.logit_cap);
         sv[i] = base + c < end ? s : NEG_INF;
@@ -563,6 +585,17 @@ static int ring_vmode(const RingParams& p, bool vshared) {
   return -1;
 }
 
+// softmax + P.V over given scores: the value rows are the C stream
+template <typename T>
+static int launch_ring_given_dt(const RingParams& p, int batch, hipStream_t st) {
+  const int nhb = p.hq <= 16 ? 1 : 2;
+#define XKV_RING_GIVEN(NHB, DN) \
+  if (nhb == NHB && p.dn == DN) return launch_ring_t<T, 32, NHB, false, DN, false, RING_VGIVEN>(p, batch, st);
+  XKV_RING_GIVEN(1, 512) XKV_RING_GIVEN(2, 512) XKV_RING_GIVEN(1, 384) XKV_RING_GIVEN(2, 384) XKV_RING_GIVEN(1, 256) XKV_RING_GIVEN(2, 256)
+#undef XKV_RING_GIVEN
+  return XKV_EUNSUPPORTED;
+}
+
 template <typename T>
 static int launch_ring_dt(const RingParams& p, int batch, bool vshared, hipStream_t st) {
   const int hg = p.hq / p.groups, vm = ring_vmode(p, vshared);
@@ -621,6 +654,10 @@ bool ring_eligible(const RingParams& p, bool vshared) {
   if (p.sCl < p.dn || (r && p.sRl < 64) || (vm == RING_VDISTINCT && p.sVl < p.dv)) return false;
   if (vm == RING_VDISTINCT && p.dn == 512 && !lo && p.dv != 512) return false;
   return true;
+}
+
+int launch_ring_given(const RingParams& p, int batch, int dtype, hipStream_t st) {
+  return dtype == XKV_BF16 ? launch_ring_given_dt<__bf16>(p, batch, st) : launch_ring_given_dt<_Float16>(p, batch, st);
 }
 
 int launch_ring(const RingParams& p, int batch, bool vshared, int dtype, hipStream_t st) {

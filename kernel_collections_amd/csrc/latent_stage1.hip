@@ -430,3 +430,31 @@ extern "C" int xkv_latent_stage1(xkv_q_operand qn, const void* qn_lo, xkv_q_oper
     return hg <= 16 ? dispatch_latent<__bf16, 1>(p, batch, vshared, st) : dispatch_latent<__bf16, 2>(p, batch, vshared, st);
   return hg <= 16 ? dispatch_latent<_Float16, 1>(p, batch, vshared, st) : dispatch_latent<_Float16, 2>(p, batch, vshared, st);
 }
+
+extern "C" int xkv_softmax_pv_stage1(const float* scores, xkv_kv_operand V, float* partial, float* lse,
+                                     const int32_t* num_kv_splits, const int32_t* kv_lens, int batch, int hq, int kv_len,
+                                     int max_splits, int split_cap_tokens, const int32_t* split_plan, int dtype, void* stream) {
+  if (!scores || !V.ptr || !partial || !lse || !num_kv_splits || batch <= 0 || hq <= 0 || kv_len <= 0 || max_splits <= 0)
+    return XKV_EINVAL;
+  if (split_cap_tokens < 0 || (split_cap_tokens > 0 && max_splits < cdiv(kv_len, split_cap_tokens))) return XKV_EINVAL;
+  if (split_plan && split_cap_tokens <= 0) return XKV_EINVAL;
+  if (dtype != XKV_BF16 && dtype != XKV_F16) return XKV_EDTYPE;
+  if (hq > 32 || (V.dim != 512 && V.dim != 384 && V.dim != 256) || V.stride_h != 0 || V.stride_l < V.dim || (kv_len & 3))
+    return XKV_EUNSUPPORTED;
+  if (!aligned8(V.stride_b) || !aligned8(V.stride_l) || !ptr16(V.ptr) || !ptr16(scores)) return XKV_EALIGN;
+  LatentParams p;
+  p.qn = nullptr; p.qn_lo = nullptr; p.qr = nullptr;
+  p.C = V.ptr; p.R = nullptr; p.V = V.ptr;
+  p.sCb = V.stride_b; p.sCl = V.stride_l; p.sCh = 0;
+  p.sRb = p.sRl = p.sRh = 0;
+  p.sVb = V.stride_b; p.sVl = V.stride_l; p.sVh = 0;
+  p.dn = V.dim; p.dr = 0; p.dv = V.dim;
+  p.partial = partial; p.lse = lse; p.scores = const_cast<float*>(scores); p.scores_dtype = XKV_F32;
+  p.num_splits = num_kv_splits; p.kv_lens = kv_lens;
+  p.hq = hq; p.groups = 1; p.kv_len = kv_len; p.max_splits = max_splits; p.split_cap = split_cap_tokens;
+  p.split_plan = split_plan;
+  p.total_wg = batch * max_splits;
+  p.sm_scale = 1.f; p.logit_cap = 0.f;
+  p.heads_in_row = 0;
+  return launch_ring_given(p, batch, dtype, (hipStream_t)stream);
+}

@@ -69,6 +69,10 @@ def decode_k_only(q, k_A, k_B, v_buffer, o, num_kv_splits, max_kv_splits, sm_sca
     return ops.merge_stage2(partial, lse, o, None, splits, lens, batch, hq, hq, kv_len, S)
 
 
+# key ranks at which fused RoPE decode with a value basis of its own runs as two passes (scores, then softmax + P.v_A)
+TWO_PASS_KEY_RANKS = (512, 384)   # at rank 256 the two forms tie
+
+
 def decode_rope(q_pe, k_A, k_B, v_A, v_B, o, num_kv_splits, max_kv_splits, sm_scale, theta, sin_cos,
                 pos_offset=0, kv_lens=None):
     """K = RoPE(k_A @ k_B) rebuilt and rotated in registers, V factorised."""
@@ -93,6 +97,20 @@ def decode_rope(q_pe, k_A, k_B, v_A, v_B, o, num_kv_splits, max_kv_splits, sm_sc
         assert sin_cos.shape == (kv_len, d), "sin_cos must be [kv_len, head_dim]"
         if sin_cos.dtype != q_pe.dtype or sin_cos.stride(-1) != 1:
             sin_cos = sin_cos.to(q_pe.dtype).contiguous()
+    same_basis = (v_A.data_ptr() == k_A.data_ptr() and v_A.shape == k_A.shape and v_A.stride() == k_A.stride())
+    if (not same_basis and k_A.shape[-1] in TWO_PASS_KEY_RANKS and sin_cos is None and hq // hkv <= 8 and hq <= 32
+            and rank_v in (256, 384, 512) and kv_len % 4 == 0 and ops.USE_RECON_WORKSPACE):
+        # A value basis of its own: two passes.  The scores-only form of the reconstruction kernel runs at the rate of the
+        # shared-basis fused kernel (one row stream, no P.A); softmax and P.v_A then stream v_A once for all heads at HBM
+        # rate.  Fused into one kernel, the second row stream costs more than the 2 x 4 bytes per score this moves.
+        scores = torch.empty((batch, hq, kv_len), dtype=torch.float32, device=q_pe.device)
+        ops.recon_stage1(q3, k_A, k_B, None, None, None, scores, splits, lens, batch, hq, hkv, kv_len, S,
+                         float(sm_scale), True, inv, int(pos_offset), None)
+        S2 = ops.latent_splits(batch, 1, kv_len, rank_v, absorbed=True)
+        splits2 = ops.uniform_splits(batch, S2, q_pe.device)
+        partial, lse = ops.workspaces(batch, hq, S2, rank_v, q_pe.device)
+        ops.softmax_pv_stage1(scores, v_A, partial, lse, splits2, lens, batch, hq, kv_len, S2, q_pe.dtype)
+        return ops.merge_stage2(partial, lse, o, v_B, splits2, lens, batch, hq, hkv, kv_len, S2)
     partial, lse = ops.workspaces(batch, hq, S, rank_v, q_pe.device)
     ops.recon_stage1(q3, k_A, k_B, v_A, partial, lse, None, splits, lens, batch, hq, hkv, kv_len, S,
                      float(sm_scale), True, inv, int(pos_offset), sin_cos)

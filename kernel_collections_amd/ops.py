@@ -188,6 +188,17 @@ def latent_stage1(qn, qn_lo, qr, C, R, V, partial, lse, scores, num_kv_splits, k
         c_float(sm_scale), c_float(logit_cap), dtype_code(qn.dtype), stream_ptr(qn)), "xkv_latent_stage1")
 
 
+def softmax_pv_stage1(scores, V, partial, lse, num_kv_splits, kv_lens, batch, hq, kv_len, max_splits, dtype,
+                      split_cap=0, split_plan=None):
+    """Stage 1 over given scores (fp32 ``[batch, hq, kv_len]``, already scaled): online softmax and ``P @ V`` per split, with V
+    ``[batch, kv_len, dv]`` one row per token for every head.  `dtype`: the 16-bit type of V (and of the rounded weights)."""
+    v = V.reshape(V.shape[0], V.shape[1], V.shape[-1]) if V.dim() == 4 else V
+    check(_lib.lib().xkv_softmax_pv_stage1(
+        ptr(scores), kv_operand(v, v.stride(0), v.stride(1), 0, v.shape[-1]), ptr(partial), ptr(lse), ptr(num_kv_splits),
+        ptr(kv_lens), batch, hq, kv_len, max_splits, int(split_cap), ptr(split_plan), dtype_code(dtype), stream_ptr(scores)),
+        "xkv_softmax_pv_stage1")
+
+
 def recon_stage1(q3, kA, kB, vA, partial, lse, scores, num_kv_splits, kv_lens, batch, hq, hkv, kv_len, max_splits,
                  sm_scale, rope, inv_freq, pos_offset, sin_cos):
     a_op = kv_operand(kA, kA.stride(0), kA.stride(1), 0, kA.shape[-1])

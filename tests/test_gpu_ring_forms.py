@@ -115,3 +115,25 @@ def test_per_head_value_forms(dev, dtype, hq):
     for dn in (512, 384, 256):                                              # absorbed keys, plain per-head values
         run_form(dev, dtype, hq=hq, dn=dn, lo=True, rope=False, mode="heads", dv=128, lens=LENS, S=SPLITS)
     run_form(dev, dtype, hq=hq, dn=128, lo=False, rope=False, mode="heads", dv=128, lens=LENS, S=SPLITS, heads_in_row=8)   # plain GQA
+
+
+@pytest.mark.parametrize("dtype", [BF, FP], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("hq", [8, 32], ids=["one_head_block", "two_head_blocks"])
+def test_softmax_pv_over_given_scores(dev, dtype, hq):
+    """xkv_softmax_pv_stage1 + merge against torch: scores are an input (peaked: sigma 6), values one row per token."""
+    lens, S = [644, 516, 32], 3
+    b, L = len(lens), 644
+    for dv in (512, 384, 256):
+        scores = draw((b, hq, L), 6.0, torch.float32, dev, 11)
+        V = draw((b, L, dv), 1.0, dtype, dev, 12)
+        splits = torch.full((b,), S, dtype=torch.int32, device=dev)
+        kl = torch.tensor(lens, dtype=torch.int32, device=dev)
+        partial, lse = ops.workspaces(b, hq, S, dv, dev)
+        ops.softmax_pv_stage1(scores, V, partial, lse, splits, kl, b, hq, L, S, dtype)
+        o = torch.empty((b, hq, dv), dtype=dtype, device=dev)
+        ops.merge_stage2(partial, lse, o, None, splits, kl, b, hq, hq, L, S)
+        for i, n in enumerate(lens):
+            p = torch.softmax(scores[i, :, :n], dim=-1).to(dtype).float()
+            ref = p @ V[i, :n].float()
+            err = max_abs(o[i].float().cpu(), ref.cpu())
+            assert err <= OUT_ATOL, f"given scores hq{hq} dv{dv} {dtype}: sequence {i}: max abs err {err:.3e}"
