@@ -67,7 +67,7 @@ struct RingShape {
   static constexpr int HB = 16 * NHB;
   static constexpr int CROW = DN * 2 + 16;                 // padded C row (bytes)
   static constexpr int CBYTES = TN * CROW;
-  static constexpr int RBYTES = HAS_R ? TN * 128 : 0;
+  static constexpr int RBYTES = (HAS_R || VMODE == RING_VGIVEN) ? TN * 128 : 0;   // RoPE-key chunks, or a tile of given scores
   static constexpr int VROW = DVW * 2 + 16;                // padded V row (distinct-V mode)
   static constexpr int VBYTES = (VMODE == RING_VDISTINCT || VMODE == RING_VHEADS) ? TN * VROW : 0;
   static constexpr int SLOT = CBYTES + RBYTES + VBYTES;
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
   // waves 4..7 move the tile rows; each brings TN/4 rows of C (and V) and two 16-byte chunks of every RoPE-key row
   constexpr int QD = RING_QD;
   constexpr int RPW = TN / 4;                     // rows per loader wave per tile
-  constexpr int LPT = RPW * IPR + (HAS_R ? 1 : 0) + (V2 ? RPW * VIPR : 0);   // loads per loader wave per tile
+  constexpr int LPT = RPW * IPR + ((HAS_R || GIVEN) ? 1 : 0) + (V2 ? RPW * VIPR : 0);   // loads per loader wave per tile
   static_assert((QD - 1) * LPT <= 63, "vmcnt holds 6 bits");
   constexpr int DV = (VMODE == RING_VSHARED || GIVEN) ? DN : VHEADS ? RING_DVH : DVW;   // value features of an output row
   constexpr int NVB = VHEADS ? RING_DVH / 16 : DV / 64;   // 16-feature blocks per wave (per kv head under VHEADS)
@@ -196,6 +196,13 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
         tok = tok < last ? tok : last;
         q[n] = ring_ldg(Rb + (int64_t)tok * rrow_bytes + (2 * iw + (lane >> 5)) * 16);
       }
+      if (GIVEN) {                       // given scores: head rows 8 iw .. +8 of the tile, 128 bytes (32 tokens) each
+        int row = 8 * iw + (lane >> 3);
+        row = row < hg ? row : hg - 1;
+        int tok = base + 4 * (lane & 7);
+        tok = tok + 4 <= p.kv_len ? tok : p.kv_len - 4;   // pieces past the buffer's row end: any in-bounds piece (masked later)
+        q[n] = ring_ldg(reinterpret_cast<const float*>(p.scores) + ((int64_t)b * p.hq + h0 + row) * p.kv_len + tok);
+      }
     };
     auto hand_on = [&](int t, u32x4 (&q)[LPT]) {   // the oldest tile of the queue: QD-1 younger ones stay in flight
       unsigned char* slot = ring + (t % RSLOT) * SLOT + lane_off;
@@ -214,7 +221,7 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
             if (DVW >= 512 || lane < DVW / 8) st16(slot + CBYTES + S::RBYTES + (iw * RPW + r) * VROW + c * 1024, q[n]);
         }
       }
-      if (HAS_R) st16(slot + CBYTES + iw * 1024, q[n]);
+      if (HAS_R || GIVEN) st16(slot + CBYTES + iw * 1024, q[n]);   // scores: [32 head rows][32 tokens] fp32, row-major
     };
     // Iteration j: tile j - QD leaves the queue for the ring (its slot was released by barrier A of the tile before it) and
     // tile j enters the queue in its place, so the look-ahead lives in the queue and a tile is waited for only when the
@@ -234,7 +241,7 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
           }
           if (j == 1 && S::qst(LO)) __syncthreads();   // the compute waves' barrier between staging the query rows and reading them
           if (k >= 1) {
-            __syncthreads();                           // B of tile k-1
+            if (!GIVEN) __syncthreads();               // B of tile k-1 (given scores: there is no QK phase to wait for)
             if (!SCORES) __syncthreads();              // C of tile k-1
           }
         }
@@ -350,17 +357,6 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
         if (LO) asm volatile("" : "+v"(qlo[k][hb]));
       }
   }
-  // Given scores: thread -> 4 tokens of one head row of the tile (8 threads per row), fetched one tile ahead into registers.
-  const int gv_row = tid >> 3, gv_c0 = (tid & 7) * 4;
-  const bool gv_active = GIVEN && gv_row < HB;
-  auto given_tile = [&](int t) -> f32x4 {
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    const int tok = start + t * TN + gv_c0;
-    if (gv_active && gv_row < hg && t < ntiles && tok + 4 <= p.kv_len)    // kv_len % 4 == 0: whole 16-byte pieces or nothing
-      v = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.scores) + ((int64_t)b * p.hq + h0 + gv_row) * p.kv_len + tok);
-    return v;
-  };
-  f32x4 gv_next = given_tile(0);
 
   // ---- running state ---------------------------------------------------------------------------------------------
   const int srow = tid / TPH, ssub = tid % TPH;
@@ -379,9 +375,7 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
     const int base = start + t * TN;
 
     // ---- QK: partial scores of token block tb over this wave's k-range -------------------------------------------
-    if constexpr (GIVEN) {               // the scores are an input: this tile's into the first partial plane, the next tile's on their way
-      if (gv_active) *reinterpret_cast<f32x4*>(s_part + gv_row * SP + gv_c0) = gv_next;
-      gv_next = given_tile(t + 1);
+    if constexpr (GIVEN) {               // the scores are an input: the loader waves put the tile's beside its value rows
     } else {
       f32x4 sacc[NHB];
 #pragma unroll
@@ -404,7 +398,7 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
       for (int hb = 0; hb < NHB; ++hb)
         *reinterpret_cast<f32x4*>(s_part + (kh * HB + hb * 16 + n16) * SP + tb * 16 + 4 * g4) = sacc[hb];
     }
-    __syncthreads();                  // B: the k-range partials of every head row are visible
+    if (!GIVEN) __syncthreads();      // B: the k-range partials of every head row are visible
 
     if (SCORES) {
       // thread -> 4 tokens (16 bytes) of a head row, TN/4 consecutive lanes per row: every store instruction writes whole
@@ -446,8 +440,12 @@ __global__ __launch_bounds__(512) void latent_ring_kernel(const RingParams p) {
       for (int i = 0; i < TPT; ++i) {
         const int c = ssub * TPT + i;
         float s = 0.f;
+        if constexpr (GIVEN) {
+          s = reinterpret_cast<const float*>(slot + CBYTES)[srow * TN + c];
+        } else {
 #pragma unroll
-        for (int kr = 0; kr < (GIVEN ? 1 : KSPLIT); ++kr) s += s_part[(kr * HB + srow) * SP + c];
+          for (int kr = 0; kr < KSPLIT; ++kr) s += s_part[(kr * HB + srow) * SP + c];
+        }
         s *= p.sm_scale;
         if (p.logit_cap > 0.f) s = p.logit_cap * tanhf(s / p.logit_cap);
         sv[i] = base + c < end ? s : NEG_INF;
