@@ -230,9 +230,17 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
 
   // ---- in-tile rotation table: accumulator registers r and r + 8 of lane (token n32, g2) are the two members of pair
   // j = 16 dq + 8 (r / 4) + 4 g2 + r % 4 ---------------------------------------------------------------------------------
-  float ci[8], si[8];
+  // kept in fp16, two registers per VGPR: the rotation runs in packed fp16 (see there)
+  typedef _Float16 rot2 __attribute__((ext_vector_type(2)));
+  rot2 ch[4], sh[4];
 #pragma unroll
-  for (int r = 0; r < 8; ++r) sincosf((float)n32 * p.inv_freq[16 * dq + 8 * (r >> 2) + 4 * g2 + (r & 3)], &si[r], &ci[r]);
+  for (int r = 0; r < 8; r += 2) {
+    float c0, s0, c1, s1;
+    sincosf((float)n32 * p.inv_freq[16 * dq + 8 * (r >> 2) + 4 * g2 + (r & 3)], &s0, &c0);
+    sincosf((float)n32 * p.inv_freq[16 * dq + 8 * ((r + 1) >> 2) + 4 * g2 + ((r + 1) & 3)], &s1, &c1);
+    ch[r >> 1] = rot2{(_Float16)c0, (_Float16)c1};
+    sh[r >> 1] = rot2{(_Float16)s0, (_Float16)s1};
+  }
 
   // ---- query-side base rotation: thread -> (head slot = wave, pair j = lane) -------------------------------------------
   float q0 = 0.f, q1 = 0.f;
@@ -321,13 +329,14 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
     f32x16 sacc;
 #pragma unroll
     for (int ks = 0; ks < KA; ++ks) {
-      if (ks < 4) {              // two pairs of the rotation per group: registers r and r + 8
-#pragma unroll
-        for (int r = 2 * ks; r < 2 * ks + 2; ++r) {
-          const int o = r >> 2, e = r & 3;
-          kop[o][e] = from_f32<sc_t>(kc[r] * ci[r] - kc[r + 8] * si[r]);
-          kop[o][4 + e] = from_f32<sc_t>(kc[r + 8] * ci[r] + kc[r] * si[r]);
-        }
+      if (ks < 4) {              // two pairs of the rotation per group: registers r, r + 1 and their partners r + 8, r + 9
+        // packed fp16 (v_pk_mul_f16 / v_pk_fma_f16): partial key sums and cos / sin rounded to fp16 first, as the
+        // reference does (fp16 accumulators and fp16 cos / sin, flash_recontruction/qAB/v1.py:59-77)
+        const int r = 2 * ks, o = r >> 2, e = r & 3;
+        const rot2 a = {(_Float16)kc[r], (_Float16)kc[r + 1]}, bb = {(_Float16)kc[r + 8], (_Float16)kc[r + 9]};
+        const rot2 lo2 = a * ch[ks] - bb * sh[ks], hi2 = bb * ch[ks] + a * sh[ks];
+        kop[o][e] = lo2[0]; kop[o][e + 1] = lo2[1];
+        kop[o][4 + e] = hi2[0]; kop[o][5 + e] = hi2[1];
       }
       if (ks + PF < NKS) fr[ks + PF] = tile_frag(t + 1, ks + PF);
       kn = Elem<T>::mfma32(breg[ks], fr[ks], ks == 0 ? z16 : kn);

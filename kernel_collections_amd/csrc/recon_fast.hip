@@ -177,11 +177,15 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   }
 
   // ---- in-tile rotation table: accumulator register r of lane (token n32, g2) is pair j = 32 dq + 8 (r/4) + 4 g2 + r%4 --
-  float ci[16], si[16];
+  typedef _Float16 rot2 __attribute__((ext_vector_type(2)));
+  rot2 ch[8], sh[8];     // cos / sin of registers 2k, 2k+1, in fp16 (8 + 8 VGPRs)
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int j = 32 * dq + 8 * (r >> 2) + 4 * g2 + (r & 3);
-    sincosf((float)n32 * p.inv_freq[j], &si[r], &ci[r]);
+  for (int r = 0; r < 16; r += 2) {
+    float c0, s0, c1, s1;
+    sincosf((float)n32 * p.inv_freq[32 * dq + 8 * (r >> 2) + 4 * g2 + (r & 3)], &s0, &c0);
+    sincosf((float)n32 * p.inv_freq[32 * dq + 8 * ((r + 1) >> 2) + 4 * g2 + ((r + 1) & 3)], &s1, &c1);
+    ch[r >> 1] = rot2{(_Float16)c0, (_Float16)c1};
+    sh[r >> 1] = rot2{(_Float16)s0, (_Float16)s1};
   }
 
   // ---- query-side base rotation: thread -> pair j = lane, head slots wave and wave + 4 ---------------------------------
@@ -333,13 +337,19 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
           }
         }
         if (DO_PREV) {
-          sc_vec8 kop;
+          // The rotation runs in packed fp16, two pairs per instruction (v_pk_mul_f16 / v_pk_fma_f16): the partial key sums
+          // and the in-tile cos / sin are rounded to fp16 first, as the reference does (fp16 accumulators and fp16 cos / sin,
+          // flash_recontruction/qAB/v1.py:59-77).  8 VALU instructions fewer per 8 rotated values than the fp32 form.
+          typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+          h2 lo2[2], hi2[2];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int r = 4 * o + e;
-            kop[e] = from_f32<sc_t>(j0[r] * ci[r] - j1[r] * si[r]);
-            kop[4 + e] = from_f32<sc_t>(j1[r] * ci[r] + j0[r] * si[r]);
+          for (int e2 = 0; e2 < 2; ++e2) {
+            const int r = 4 * o + 2 * e2;
+            const h2 a = {(_Float16)j0[r], (_Float16)j0[r + 1]}, bb = {(_Float16)j1[r], (_Float16)j1[r + 1]};
+            lo2[e2] = a * ch[2 * o + e2] - bb * sh[2 * o + e2];
+            hi2[e2] = bb * ch[2 * o + e2] + a * sh[2 * o + e2];
           }
+          const sc_vec8 kop = {lo2[0][0], lo2[0][1], lo2[1][0], lo2[1][1], hi2[0][0], hi2[0][1], hi2[1][0], hi2[1][1]};
           if (o == 0) {
             const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             sacc = Elem<sc_t>::mfma32(kop, qop[o], z);
