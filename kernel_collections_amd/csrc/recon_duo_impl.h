@@ -51,7 +51,7 @@ template <typename T> constexpr float lazy_rescale() { return std::is_same<T, _F
 #define XKV_DUO_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)   // 0x8 MFMA, 0x2 VALU, 0x100 LDS read, 0x200 LDS write
 
 // LDS budget: everything but the tile rings
-constexpr int DUO_TAIL = NW * 8 * FSP_ROW * 4 + 2 * 8 * 128 * 2 + 2 * 16 * FP_ROW * 2 + 32 * 4 + 16 * 4;
+constexpr int DUO_TAIL = NW * 8 * FSP_ROW * 4 + 2 * 8 * 128 * 2 + 2 * 16 * FP_ROW * 2 + 32 * 4 + 16 * 4 + 32 * 2;
 
 template <int RK, int RV, int MODE>
 struct DuoShape {
@@ -204,9 +204,11 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
   T* p_lds = reinterpret_cast<T*>(qhat + 2 * 8 * 128);                                          // [2][16 head slots][FP_ROW]
   float* alpha_lds = reinterpret_cast<float*>(p_lds + 2 * 16 * FP_ROW);    // [2][16]
   float* ml_lds = alpha_lds + 32;                                          // [8][2]
+  sc_t* qzero = reinterpret_cast<sc_t*>(ml_lds + 16);                      // [32] zeros: the q-dot operand of masked lanes
   const unsigned smem_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)smem;
   for (int i = tid; i < 2 * 16 * FP_ROW; i += 64 * NW) p_lds[i] = from_f32<T>(0.f);   // slots of absent heads stay zero
   if (tid < 32) alpha_lds[tid] = 1.f;
+  if (tid < 32) qzero[tid] = from_f32<sc_t>(0.f);
 
   // ---- async tile loads: wave w brings rows 4w .. 4w+3 of every tile ---------------------------------------------
   DuoStream<RK, KROW, NSK> ks_;
@@ -281,7 +283,13 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
   auto tile_frag = [&](int t, int ks) -> vec8 {
     return ld16<vec8>(kring + (t % NSK) * KTILE + n32 * KROW + ((RK / 2) * kq + 8 * g2) * 2 + ks * 32);
   };
-  const sc_t* qrow = qhat + (n32 < G ? n32 : G - 1) * 128 + (dq * 4 + g2) * 8;
+  // q-dot on v_mfma_f32_16x16x32: as its A operand, lane (n32, g2) is row n32 % 16 and k-group (n32 / 16) + 2 g2, so the two
+  // token halves of the tile land in the same 16 rows as different k-groups; the B operand keeps them apart: column c holds
+  // q^ of head c % 8 in the k-groups of token half c / 8 (lanes whose bit 4 equals bit 3) and zeros in the other two.
+  // Result: lane (c, g4), register r = score of token 16 (c / 8) + 4 g4 + r for head c % 8.
+  const bool q_live = ((lane >> 4) & 1) == ((lane >> 3) & 1);
+  const sc_t* qrow = q_live ? qhat + ((lane & 7) < G ? (lane & 7) : G - 1) * 128 + (dq * 4 + g2) * 8 : qzero;
+  const int qpar = q_live ? 8 * 128 : 0;   // q^ is double-buffered by tile parity, the zeros are not
   auto tr_read = [&](int t) {   // this wave's DV/8 value features of tile t, token-major
     if (SCORES) return;
     constexpr int VR = V2 ? VROW : KROW;
@@ -323,10 +331,10 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
     vec8 fr[NKS];
 #pragma unroll
     for (int i = 0; i < PF; ++i) fr[i] = tile_frag(t + 1, i);
-    const sc_t* qr = qrow + PAR * (8 * 128);
+    const sc_t* qr = qrow + PAR * qpar;
     const sc_vec8 qop0 = ld16<sc_vec8>(qr), qop1 = ld16<sc_vec8>(qr + 16);
     sc_vec8 kop[2];
-    f32x16 sacc;
+    f32x4 sacc;
 #pragma unroll
     for (int ks = 0; ks < KA; ++ks) {
       if (ks < 4) {              // two pairs of the rotation per group: registers r, r + 1 and their partners r + 8, r + 9
@@ -340,20 +348,16 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
       }
       if (ks + PF < NKS) fr[ks + PF] = tile_frag(t + 1, ks + PF);
       kn = Elem<T>::mfma32(breg[ks], fr[ks], ks == 0 ? z16 : kn);
-      if (ks == 1) sacc = Elem<sc_t>::mfma32(kop[0], qop0, z16);
-      if (ks == 3) sacc = Elem<sc_t>::mfma32(kop[1], qop1, sacc);
+      if (ks == 1) sacc = Elem<sc_t>::mfma16(kop[0], qop0, f32x4{0.f, 0.f, 0.f, 0.f});
+      if (ks == 3) sacc = Elem<sc_t>::mfma16(kop[1], qop1, sacc);
       if (ks == 2) {             // scalar address work and the load issue run under the MFMAs already in the pipe
         XKV_DUO_FENCE();
         ks_.issue(end, last, wave, lane);          // key tile t + KAHEAD, into the slot freed at the last barrier
         if (V2) vs_.issue(end, last, wave, lane);  // value tile t + VAHEAD
       }
-      if (ks == (KA > 5 ? 5 : KA - 1)) {   // lane (n32 = head, g2): register r of sacc = token 8 (r/4) + 4 g2 + r%4
-        if (n32 < G) {
-          float* dst = s_part + (wave * 8 + n32) * FSP_ROW + 4 * g2;
-#pragma unroll
-          for (int qd = 0; qd < 4; ++qd)
-            *reinterpret_cast<f32x4*>(dst + 8 * qd) = f32x4{sacc[4 * qd], sacc[4 * qd + 1], sacc[4 * qd + 2], sacc[4 * qd + 3]};
-        }
+      if (ks == (KA > 5 ? 5 : KA - 1)) {
+        if ((n16 & 7) < G)
+          *reinterpret_cast<f32x4*>(s_part + (wave * 8 + (n16 & 7)) * FSP_ROW + 16 * (n16 >> 3) + 4 * g4) = sacc;
       }
       XKV_DUO_FENCE();
     }

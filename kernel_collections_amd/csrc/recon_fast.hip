@@ -131,9 +131,11 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   T* p_lds = reinterpret_cast<T*>(qhat + 2 * 8 * 128);                                          // [16 head slots][FP_ROW]
   float* alpha_lds = reinterpret_cast<float*>(p_lds + 16 * FP_ROW);        // [16]
   float* ml_lds = alpha_lds + 16;                                          // [8][2]
+  sc_t* qzero = reinterpret_cast<sc_t*>(ml_lds + 16);                      // [128] zeros: the q-dot operand of masked lanes
   const unsigned ring_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)ring;
   for (int i = tid; i < 16 * FP_ROW; i += 256) p_lds[i] = from_f32<T>(0.f);   // slots of absent heads stay zero
   if (tid < 16) alpha_lds[tid] = 1.f;
+  if (tid < 128) qzero[tid] = from_f32<sc_t>(0.f);
 
   // ---- async tile loads: wave w brings rows 8w .. 8w+7, one 1 KiB row per instruction ------------------------------
   // Scalar row pointers advance by adds only; the clamped form is needed only where a tile crosses the split end.
@@ -222,6 +224,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     sc_t* dst = qhat + (t & 1) * (8 * 128) + wave * 128 + qpos;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
+      if (i == 1 && G <= 4) break;   // head slots 4..7 are absent: nothing reads their rows
       dst[i * 512] = from_f32<sc_t>(q0[i] * qcb + q1[i] * qsb);
       dst[i * 512 + 4] = from_f32<sc_t>(q1[i] * qcb - q0[i] * qsb);
     }
@@ -282,6 +285,12 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     alpha_lds[sm_head] = alpha;
   };
 
+  // ---- q-dot B operand source: lanes whose token half (lane bit 4) matches their column's (lane bit 3) read q^ of head
+  // lane % 8 (absent heads: the last one; their columns are not stored), the others read zeros ------------------------------
+  const bool q_live = ((lane >> 4) & 1) == ((lane >> 3) & 1);
+  const sc_t* qsrc = q_live ? qhat + ((lane & 7) < G ? (lane & 7) : G - 1) * 128 + (dq * 2 + g2) * 8 : qzero;
+  const int qpar = q_live ? 8 * 128 : 0;   // q^ is double-buffered by tile parity, the zeros are not
+
   // ---- accumulators and loop-carried operand registers ---------------------------------------------------------------------
   f32x4 acc[8];          // P.A: wave w owns latent features 128 w .. +128
 #pragma unroll
@@ -319,7 +328,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     // waves queue on the LDS pipe right after every barrier.
     // ---- part 1 ----------------------------------------------------------------------------------------------------------
     {
-      f32x16 sacc;
+      f32x4 sacc;
 #pragma unroll
       for (int o = 0; o < 4; ++o) {
         if (DO_R) {
@@ -350,12 +359,11 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
             hi2[e2] = bb * ch[2 * o + e2] + a * sh[2 * o + e2];
           }
           const sc_vec8 kop = {lo2[0][0], lo2[0][1], lo2[1][0], lo2[1][1], hi2[0][0], hi2[0][1], hi2[1][0], hi2[1][1]};
-          if (o == 0) {
-            const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            sacc = Elem<sc_t>::mfma32(kop, qop[o], z);
-          } else {
-            sacc = Elem<sc_t>::mfma32(kop, qop[o], sacc);
-          }
+          // q-dot on v_mfma_f32_16x16x32: as its A operand, lane (n32, g2) is row n32 % 16 and k-group (n32 / 16) + 2 g2, so
+          // the two token halves of the tile land in the same 16 rows as different k-groups; the B operand keeps them apart:
+          // column c holds q^ of head c % 8 in the k-groups of token half c / 8 and zeros in the other two.  Result: lane
+          // (c, g4), register r = score of token 16 (c / 8) + 4 g4 + r for head c % 8.
+          sacc = Elem<sc_t>::mfma16(kop, qop[o], o == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : sacc);
         }
         if (DO_R && DO_PREV) {   // three reconstruction MFMAs dealt out among the rotation's VALU work, then the q-dot
           XKV_SGB(0x8, 1); XKV_SGB(0x2, 7);
@@ -365,13 +373,8 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
         }
         XKV_FENCE();
       }
-      // lane (n32 = head, g2): register r of sacc = token 8 (r/4) + 4 g2 + r%4
-      if (DO_PREV && n32 < G) {
-        float* dst = s_part + (wave * 8 + n32) * FSP_ROW + 4 * g2;
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd)
-          *reinterpret_cast<f32x4*>(dst + 8 * qd) = f32x4{sacc[4 * qd], sacc[4 * qd + 1], sacc[4 * qd + 2], sacc[4 * qd + 3]};
-      }
+      if (DO_PREV && (n16 & 7) < G)
+        *reinterpret_cast<f32x4*>(s_part + (wave * 8 + (n16 & 7)) * FSP_ROW + 16 * (n16 >> 3) + 4 * g4) = sacc;
     }
     __syncthreads();        // B_b: partial scores of tile i-1 are visible
     // ---- part 2 ----------------------------------------------------------------------------------------------------------
@@ -422,7 +425,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     vec8 pb;
     vec8 at_next[6];
     sc_vec8 qop_next[4];
-    const sc_t* qrow = qhat + (i & 1) * (8 * 128) + (n32 < G ? n32 : G - 1) * 128 + (dq * 2 + g2) * 8;
+    const sc_t* qrow = qsrc + (i & 1) * qpar;
     auto pv_step = [&](int mb) {
       if (SCORES) return;
       vec8 a = __builtin_bit_cast(vec8, (s16x8f)__builtin_shufflevector(tr[2 * mb], tr[2 * mb + 1], 0, 1, 2, 3, 4, 5, 6, 7));
@@ -507,7 +510,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   }
 }
 
-constexpr size_t FAST_SHM = (size_t)FRING * FTILE + 4 * 8 * FSP_ROW * 4 + 2 * 8 * 128 * 2 + 16 * FP_ROW * 2 + 16 * 4 + 16 * 4;
+constexpr size_t FAST_SHM = (size_t)FRING * FTILE + 4 * 8 * FSP_ROW * 4 + 2 * 8 * 128 * 2 + 16 * FP_ROW * 2 + 16 * 4 + 16 * 4 + 128 * 2;
 
 template <typename T>
 int launch_recon_fast_t(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, hipStream_t st) {
