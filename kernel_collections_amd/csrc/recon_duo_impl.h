@@ -258,6 +258,7 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
   float qc32, qs32, qcb = 1.f, qsb = 0.f;   // (qcb, qsb): base rotation of the tile whose q^ is written next
   sincosf((float)FT * qinv, &qs32, &qc32);
   auto write_qhat = [&](int t) {   // q^ for tile t = R(-base(t)) q, into buffer t & 1
+    if (wave >= G) return;         // absent head slot: nothing reads its row
     if ((t & 31) == 0)             // the base advances by angle addition; every 32 tiles it is range-reduced afresh
       sincosf((float)(p.pos_offset + start + (int64_t)t * FT) * qinv, &qsb, &qcb);
     sc_t* dst = qhat + (t & 1) * (8 * 128) + wave * 128 + qpos;

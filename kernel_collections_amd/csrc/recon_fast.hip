@@ -18,18 +18,18 @@
 // Pipeline.  A wave issues instructions in order, so MFMA time and VALU time only overlap when independent
 // work is interleaved in its instruction stream.  Iteration i therefore runs the 16 reconstruction MFMA steps of
 // tile i (accumulating into one of two key-accumulator sets) in three parts, interleaved with what tile i-1 still
-// needs: part 1 (steps 0..5) rotates tile i-1's partial keys (the other accumulator set), dots them with q^ and
-// stores the partial scores, while the pair-index threads write q^ for tile i; barrier; part 2 (steps 6..10)
-// issues the loads of tile i+2, runs the softmax of tile i-1 (one owner lane group per head: no redundant work)
-// and publishes P and the rescale factor through LDS; barrier; part 3 (steps 11..15) accumulates P.A for tile
-// i-1, each wave owning 128 latent features, the token-major operand coming from ds_read_b64_tr_b16, and
-// prefetches the first LDS operands of tile i+1.  Two barriers per tile separate the parts.
-// The softmax reference only moves when a tile maximum exceeds it by 16 (lazy rescaling), so the P.A
-// accumulators are almost never rescaled.
+// needs: part 1 (steps 0..5) rotates tile i-1's partial keys (the other accumulator set) in packed fp16, dots them
+// with q^ on v_mfma_f32_16x16x32 and stores the partial scores; barrier; part 2 (steps 6..10) runs the softmax of
+// tile i-1 (one owner lane group per head: no redundant work), publishes P and the rescale factor through LDS and
+// reads tile i-1 transposed for P.A; barrier; part 3 (steps 11..15) accumulates P.A for tile i-1, each wave owning
+// 128 latent features, issues the loads of tile i+3 into the slot tile i-1 has left (one load behind each MFMA),
+// writes q^ for tile i+1 and prefetches the first LDS operands of tile i+1.  Two barriers per tile separate the parts.
+// The softmax reference only moves when a tile maximum exceeds it by 16 (8 for fp16 operands: lazy rescaling), so the
+// P.A accumulators are almost never rescaled.
 //
-// Tiles stream through a 4-slot LDS ring filled by direct-to-LDS loads issued two tiles ahead.  Those loads
+// Tiles stream through a 4-slot LDS ring filled by direct-to-LDS loads issued three tiles ahead.  Those loads
 // are inline asm so that the compiler's wait-count pass does not serialise them against every LDS read;
-// completion is tracked by hand (s_waitcnt vmcnt(8): the 8 loads of the next tile may still be in flight).
+// completion is tracked by hand (s_waitcnt vmcnt(8): the 8 loads of the next tile but one may still be in flight).
 #include "xkv_common.h"
 #include "recon_fast.h"
 #include <type_traits>
@@ -59,18 +59,14 @@ __device__ __forceinline__ void async_row16(const void* row_base, unsigned lane_
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_off), "s"(row_base)
                : "memory", "m0");
 }
-// Four rows with one M0 / base pair: the instruction offset r * FROW moves the LDS address AND the global address, so the
-// per-row lane offsets voff[r] = lane * 16 + 128 + r * (row_bytes - FROW) (base = first row - 128 bytes) put row r of the
-// tile at global row r.  (FROW must stay below 4096 / 3 for the 13-bit offset field.)
-__device__ __forceinline__ void async_rows4(const void* base_m128, unsigned v0, unsigned v1, unsigned v2, unsigned v3,
-                                            unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-               "global_load_lds_dwordx4 %1, %5\n\t"
-               "global_load_lds_dwordx4 %2, %5 offset:1040\n\t"
-               "global_load_lds_dwordx4 %3, %5 offset:2080\n\t"
-               "global_load_lds_dwordx4 %4, %5 offset:3120"
-               ::"s"(lds_addr), "v"(v0), "v"(v1), "v"(v2), "v"(v3), "s"(base_m128)
-               : "memory", "m0");
+// The instruction offset moves the LDS address AND the global address: with base = (first row of a group of four) - 128
+// bytes and per-row lane offsets voff[r] = lane * 16 + 128 + r * (row_bytes - FROW), the instruction offset r * FROW puts
+// global row r at tile row r, so the four rows of a group share one scalar base and one M0 value.  (FROW must stay below
+// 4096 / 3 for the 13-bit offset field.)
+template <int OFF>
+__device__ __forceinline__ void async_row_off(const void* base_m128, unsigned voff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
+               ::"s"(lds_addr), "v"(voff), "s"(base_m128), "n"(OFF) : "memory", "m0");
 }
 template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
@@ -145,28 +141,27 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   unsigned voff4[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) voff4[r] = lane_off + 128u + (unsigned)(r * ((int)row_bytes - FROW));
-  auto issue_rows = [&](int t, auto r0_c, auto r1_c, auto full_c) {   // rows r0 .. r1-1 of this wave's 8 rows of tile t
-    constexpr int R0 = decltype(r0_c)::value, R1 = decltype(r1_c)::value;
-    const unsigned dst = ring_lds + (unsigned)(t & (FRING - 1)) * FTILE + (unsigned)(wave * 8) * FROW;
+  // One row per call: in the loop every load sits behind an MFMA of its own (a burst of loads holds the wave's issue for
+  // about 20 cycles per instruction).  full_c: the caller knows the whole tile lies inside the split.
+  auto issue_one = [&](int t, auto r_c, auto full_c) {
+    constexpr int R = decltype(r_c)::value;
     const int tok0 = start + t * FT + wave * 8;
-    if (decltype(full_c)::value) {   // the caller knows the whole tile lies inside the split
-      static_assert(!decltype(full_c)::value || ((R1 - R0) % 4 == 0 && R0 % 4 == 0), "full tiles are issued four rows at a time");
-#pragma unroll
-      for (int r = R0; r < R1; r += 4)
-        async_rows4(Ab + (int64_t)(tok0 + r) * row_bytes - 128, voff4[0], voff4[1], voff4[2], voff4[3], dst + r * FROW);
+    if (decltype(full_c)::value) {
+      const unsigned dst = ring_lds + (unsigned)(t & (FRING - 1)) * FTILE + (unsigned)(wave * 8 + (R & ~3)) * FROW;
+      async_row_off<(R & 3) * FROW>(Ab + (int64_t)(tok0 + (R & ~3)) * row_bytes - 128, voff4[R & 3], dst);
     } else {
-#pragma unroll
-      for (int r = R0; r < R1; ++r) {
-        int tok = tok0 + r;
-        tok = tok < last ? tok : last;   // rows past the split end are masked in the softmax; keep the read in bounds
-        async_row16(Ab + (int64_t)tok * row_bytes, lane_off, dst + r * FROW);
-      }
+      int tok = tok0 + R;
+      tok = tok < last ? tok : last;   // rows past the split end are masked in the softmax; keep the read in bounds
+      async_row16(Ab + (int64_t)tok * row_bytes, lane_off, ring_lds + (unsigned)(t & (FRING - 1)) * FTILE + (unsigned)(wave * 8 + R) * FROW);
     }
   };
-  auto issue_tile = [&](int t, auto full_c) { issue_rows(t, IC<0>(), IC<8>(), full_c); };
-  issue_tile(0, IC<0>());
-  issue_tile(1, IC<0>());
-  issue_tile(2, IC<0>());
+  auto issue_tile = [&](int t) {
+    issue_one(t, IC<0>(), IC<0>()); issue_one(t, IC<1>(), IC<0>()); issue_one(t, IC<2>(), IC<0>()); issue_one(t, IC<3>(), IC<0>());
+    issue_one(t, IC<4>(), IC<0>()); issue_one(t, IC<5>(), IC<0>()); issue_one(t, IC<6>(), IC<0>()); issue_one(t, IC<7>(), IC<0>());
+  };
+  issue_tile(0);
+  issue_tile(1);
+  issue_tile(2);
 
   // ---- stationary B operands: 16 k-steps x 2 feature blocks, kept in accumulation registers ---------------------------
   vec8 breg[16][2];
@@ -441,11 +436,15 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     }
     if (DO_R) {
       at_next[0] = tile_frag(i + 1, 0);
-      recon_step(11);
+      k0 = Elem<T>::mfma32(breg[11][0], at[11], k0);
+      XKV_FENCE();
+      issue_one(i + 3, IC<0>(), full_c);
+      XKV_FENCE();
+      k1 = Elem<T>::mfma32(breg[11][1], at[11], k1);
     }
     XKV_FENCE();
-#pragma unroll
-    for (int u = 1; u < 5; ++u) {
+    auto grp = [&](auto u_c) {
+      constexpr int u = decltype(u_c)::value;
       if (DO_PREV) {
         pv_step(2 * u - 2);
         pv_step(2 * u - 1);
@@ -454,13 +453,20 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
         at_next[u] = tile_frag(i + 1, u);
         if (u == 4) at_next[5] = tile_frag(i + 1, 5);
         qop_next[u - 1] = ld16<sc_vec8>(qrow + (u - 1) * 32);
-        recon_step(11 + u);
-        if (u == 1) issue_rows(i + 3, IC<0>(), IC<4>(), full_c);   // into the ring slot of tile i-1, whose readers are done
-        if (u == 3) issue_rows(i + 3, IC<4>(), IC<8>(), full_c);
-        if (u == 4) write_qhat(i + 1);                             // buffer (i+1)&1 was last read in part 3 of iteration i-1
+        k0 = Elem<T>::mfma32(breg[11 + u][0], at[11 + u], k0);
+        XKV_FENCE();
+        issue_one(i + 3, IC<2 * u - 1>(), full_c);
+        XKV_FENCE();
+        k1 = Elem<T>::mfma32(breg[11 + u][1], at[11 + u], k1);
+        if (u < 4) {
+          XKV_FENCE();
+          issue_one(i + 3, IC<2 * u>(), full_c);
+        }
+        if (u == 4) write_qhat(i + 1);
       }
       XKV_FENCE();
-    }
+    };
+    grp(IC<1>()); grp(IC<2>()); grp(IC<3>()); grp(IC<4>());
     if (DO_R) {
 #pragma unroll
       for (int ks = 0; ks < 6; ++ks) at[ks] = at_next[ks];
