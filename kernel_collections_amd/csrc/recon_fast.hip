@@ -175,15 +175,18 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
 
   // ---- in-tile rotation table: accumulator register r of lane (token n32, g2) is pair j = 32 dq + 8 (r/4) + 4 g2 + r%4 --
   typedef _Float16 rot2 __attribute__((ext_vector_type(2)));
-  rot2 ch[8], sh[8];     // cos / sin of registers 2k, 2k+1, in fp16 (8 + 8 VGPRs)
+  // Two tables: the query-side base is that of an EVEN tile and serves the odd tile after it too, whose offsets are 32 .. 63.
+  rot2 ch[2][8], sh[2][8];     // [tile parity]: cos / sin of registers 2k, 2k+1, in fp16 (16 + 16 VGPRs)
 #pragma unroll
-  for (int r = 0; r < 16; r += 2) {
-    float c0, s0, c1, s1;
-    sincosf((float)n32 * p.inv_freq[32 * dq + 8 * (r >> 2) + 4 * g2 + (r & 3)], &s0, &c0);
-    sincosf((float)n32 * p.inv_freq[32 * dq + 8 * ((r + 1) >> 2) + 4 * g2 + ((r + 1) & 3)], &s1, &c1);
-    ch[r >> 1] = rot2{(_Float16)c0, (_Float16)c1};
-    sh[r >> 1] = rot2{(_Float16)s0, (_Float16)s1};
-  }
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      float c0, s0, c1, s1;
+      sincosf((float)(n32 + 32 * h) * p.inv_freq[32 * dq + 8 * (r >> 2) + 4 * g2 + (r & 3)], &s0, &c0);
+      sincosf((float)(n32 + 32 * h) * p.inv_freq[32 * dq + 8 * ((r + 1) >> 2) + 4 * g2 + ((r + 1) & 3)], &s1, &c1);
+      ch[h][r >> 1] = rot2{(_Float16)c0, (_Float16)c1};
+      sh[h][r >> 1] = rot2{(_Float16)s0, (_Float16)s1};
+    }
 
   // ---- query-side base rotation: thread -> pair j = lane, head slots wave and wave + 4 ---------------------------------
   float q0[2], q1[2];
@@ -203,7 +206,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   // a lane's 8 contraction values of chunk o are one 16-byte read
   const int qpos = ((((lane >> 3) & 3) * 2 + (lane >> 5)) * 2 + ((lane >> 2) & 1)) * 8 + (lane & 3);
   float qc32, qs32, qcb = 1.f, qsb = 0.f;   // (qcb, qsb): base rotation of the tile whose q^ is written next
-  sincosf((float)FT * qinv, &qs32, &qc32);
+  sincosf((float)(2 * FT) * qinv, &qs32, &qc32);   // the base advances two tiles at a time
   // The base advances by angle addition; every 32 tiles it is replaced by a freshly range-reduced value (the seed),
   // computed outside the pipeline's inner loop and swapped in with a select so that write_qhat stays branch-free.
   int seed_t = 0;
@@ -212,11 +215,11 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     seed_t = t;
     sincosf((float)(p.pos_offset + start + (int64_t)t * FT) * qinv, &seed_s, &seed_c);
   };
-  auto write_qhat = [&](int t) {   // q^ for tile t = R(-base(t)) q
+  auto write_qhat = [&](int t) {   // q^ for the even tile t and the odd one after it = R(-base(t)) q, into buffer (t / 2) & 1
     const bool sd = t == seed_t;
     qcb = sd ? seed_c : qcb;
     qsb = sd ? seed_s : qsb;
-    sc_t* dst = qhat + (t & 1) * (8 * 128) + wave * 128 + qpos;
+    sc_t* dst = qhat + ((t >> 1) & 1) * (8 * 128) + wave * 128 + qpos;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       if (i == 1 && G <= 4) break;   // head slots 4..7 are absent: nothing reads their rows
@@ -233,7 +236,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   const int sm_head = wave + 4 * ((lane >> 4) & 1);
   const int sm_row = sm_head < G ? sm_head : G - 1;
   const bool sm_valid = sm_head < G;
-  float m_ref = NEG_INF, l_run = 0.f;
+  float m_ref = NEG_INF, l_run = 0.f;   // reference maximum of the lane's head; this lane's share of the head's row sum
   f32x2 sp_v[4];
   auto softmax_read = [&]() {   // the four waves' partial scores of this lane's two tokens
     const float* sp = s_part + sm_row * FSP_ROW + 2 * n16;
@@ -273,7 +276,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       m_ref = m_new;
     }
     const float e0 = __expf(s0 - m_ref), e1 = __expf(s1 - m_ref);
-    l_run = l_run * alpha + row_reduce<false, 16>(e0 + e1);
+    l_run = l_run * alpha + (e0 + e1);   // per lane (alpha is the head's, the same in all 16): summed over the lanes once, at the end
     T* pd = p_lds + sm_head * FP_ROW + 2 * n16;
     pd[0] = from_f32<T>(sm_valid ? e0 : 0.f);
     pd[1] = from_f32<T>(sm_valid ? e1 : 0.f);
@@ -350,8 +353,8 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
           for (int e2 = 0; e2 < 2; ++e2) {
             const int r = 4 * o + 2 * e2;
             const h2 a = {(_Float16)j0[r], (_Float16)j0[r + 1]}, bb = {(_Float16)j1[r], (_Float16)j1[r + 1]};
-            lo2[e2] = a * ch[2 * o + e2] - bb * sh[2 * o + e2];
-            hi2[e2] = bb * ch[2 * o + e2] + a * sh[2 * o + e2];
+            lo2[e2] = a * ch[PAR ^ 1][2 * o + e2] - bb * sh[PAR ^ 1][2 * o + e2];   // tile i-1: parity PAR ^ 1
+            hi2[e2] = bb * ch[PAR ^ 1][2 * o + e2] + a * sh[PAR ^ 1][2 * o + e2];
           }
           const sc_vec8 kop = {lo2[0][0], lo2[0][1], lo2[1][0], lo2[1][1], hi2[0][0], hi2[0][1], hi2[1][0], hi2[1][1]};
           // q-dot on v_mfma_f32_16x16x32: as its A operand, lane (n32, g2) is row n32 % 16 and k-group (n32 / 16) + 2 g2, so
@@ -412,7 +415,10 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       wait_vmcnt<8>();      // this wave's rows of tile i+1 have landed (the 8 loads of tile i+2 may be in flight)
     } else {
       wait_vmcnt<0>();
-      if (!SCORES && sm_valid && n16 == 0) { ml_lds[2 * sm_head] = m_ref; ml_lds[2 * sm_head + 1] = l_run; }   // final state for the epilogue
+      if (!SCORES) {        // final state for the epilogue
+        const float l_head = row_reduce<false, 16>(l_run);
+        if (sm_valid && n16 == 0) { ml_lds[2 * sm_head] = m_ref; ml_lds[2 * sm_head + 1] = l_head; }
+      }
     }
     __syncthreads();        // B_c: P and rescale factors of tile i-1 are visible; tile i+1 is complete for every wave;
                             // the transposed reads of tile i-1 have returned, so its ring slot is free
@@ -420,7 +426,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     vec8 pb;
     vec8 at_next[6];
     sc_vec8 qop_next[4];
-    const sc_t* qrow = qsrc + (i & 1) * qpar;
+    const sc_t* qrow = qsrc + ((i >> 1) & 1) * qpar;   // q^ of the pair of tiles i (even) opens
     auto pv_step = [&](int mb) {
       if (SCORES) return;
       vec8 a = __builtin_bit_cast(vec8, (s16x8f)__builtin_shufflevector(tr[2 * mb], tr[2 * mb + 1], 0, 1, 2, 3, 4, 5, 6, 7));
@@ -452,7 +458,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       if (DO_R) {
         at_next[u] = tile_frag(i + 1, u);
         if (u == 4) at_next[5] = tile_frag(i + 1, 5);
-        qop_next[u - 1] = ld16<sc_vec8>(qrow + (u - 1) * 32);
+        if (PAR == 0) qop_next[u - 1] = ld16<sc_vec8>(qrow + (u - 1) * 32);   // an odd tile keeps its predecessor's
         k0 = Elem<T>::mfma32(breg[11 + u][0], at[11 + u], k0);
         XKV_FENCE();
         issue_one(i + 3, IC<2 * u - 1>(), full_c);
@@ -462,7 +468,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
           XKV_FENCE();
           issue_one(i + 3, IC<2 * u>(), full_c);
         }
-        if (u == 4) write_qhat(i + 1);
+        if (u == 4 && PAR == 1) write_qhat(i + 1);   // buffer ((i+1)/2)&1 was last read in part 3 of iteration i-3
       }
       XKV_FENCE();
     };
@@ -471,7 +477,8 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
 #pragma unroll
       for (int ks = 0; ks < 6; ++ks) at[ks] = at_next[ks];
 #pragma unroll
-      for (int o = 0; o < 4; ++o) qop[o] = qop_next[o];
+      for (int o = 0; o < 4; ++o)
+        if (PAR == 0) qop[o] = qop_next[o];
     }
   };
 
