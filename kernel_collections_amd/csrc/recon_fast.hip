@@ -432,13 +432,10 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       vec8 a = __builtin_bit_cast(vec8, (s16x8f)__builtin_shufflevector(tr[2 * mb], tr[2 * mb + 1], 0, 1, 2, 3, 4, 5, 6, 7));
       acc[mb] = Elem<T>::mfma16(a, pb, acc[mb]);
     };
+    float al = 1.f;
     if (DO_PREV && !SCORES) {
-      const float al = alpha_lds[n16];
+      al = alpha_lds[n16];
       pb = ld16<vec8>(p_lds + n16 * FP_ROW + 8 * g4);
-      if (__builtin_amdgcn_ballot_w64(al != 1.f)) {   // rare: the softmax reference moved
-#pragma unroll
-        for (int mb = 0; mb < 8; ++mb) acc[mb] *= al;
-      }
     }
     if (DO_R) {
       at_next[0] = tile_frag(i + 1, 0);
@@ -449,6 +446,12 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       k1 = Elem<T>::mfma32(breg[11][1], at[11], k1);
     }
     XKV_FENCE();
+    if (DO_PREV && !SCORES) {   // the two MFMAs above cover the LDS latency of the rescale factor this branch waits for
+      if (__builtin_amdgcn_ballot_w64(al != 1.f)) {   // rare: the softmax reference moved
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) acc[mb] *= al;
+      }
+    }
     auto grp = [&](auto u_c) {
       constexpr int u = decltype(u_c)::value;
       if (DO_PREV) {
