@@ -18,13 +18,13 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-inline-asm",
 ]
-# Per-file additions.  recon_fast.hip and the recon_duo_*.hip units: MFMA results must land in ordinary VGPRs (the RoPE / softmax VALU code reads
+# Per-file additions.  the recon_fast_*.hip and recon_duo_*.hip units: MFMA results must land in ordinary VGPRs (the RoPE / softmax VALU code reads
 # them; with accumulation-register results every value costs a v_accvgpr_read), while the stationary B operands are
 # pinned to accumulation registers by the source itself.
 _VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 EXTRA_FLAGS = {
-    "recon_fast.hip": _VGPR_FORM,
-    "recon_duo_a.hip": _VGPR_FORM, "recon_duo_b.hip": _VGPR_FORM, "recon_duo_c.hip": _VGPR_FORM,
+    "recon_fast_512.hip": _VGPR_FORM, "recon_fast_384.hip": _VGPR_FORM, "recon_fast_256.hip": _VGPR_FORM,
+    "recon_duo_b.hip": _VGPR_FORM, "recon_duo_c.hip": _VGPR_FORM,
 }
 
 

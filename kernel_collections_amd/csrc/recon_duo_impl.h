@@ -1,7 +1,7 @@
-// Fused reconstruct + RoPE + softmax + P.A stage 1 for the shapes the 4-wave kernel (recon_fast.hip) is not built for:
-// key rank 256 / 384 / 512, head_dim 128, computed RoPE angles, and either scores only, the key basis reused as the value
-// basis, or a SEPARATE value basis of rank 256 / 384 / 512 (a second row stream).  Included by the recon_duo_*.hip
-// translation units, which instantiate the shapes.
+// Fused reconstruct + RoPE + softmax + P.A stage 1 with a SEPARATE value basis (a second row stream), which the 4-wave
+// kernel (recon_fast_impl.h) is not built for: key rank 256 / 384 / 512, value rank 256 / 384 / 512, head_dim 128, computed
+// RoPE angles.  (The template also has a scores-only and a shared-basis mode; the 4-wave kernel is the faster one there and
+// the dispatcher sends those shapes to it.)  Included by the recon_duo_*.hip translation units, which instantiate the shapes.
 //
 // Work split.  One workgroup = one (batch, kv head, split), 8 wavefronts = two per SIMD.  The waves form a 2 x 4 grid
 // over (rank half kq, feature quarter dq): wave (kq, dq) keeps B[kh][RK/2 kq .. +RK/2][{16 dq .. +16} u {64 + 16 dq .. +16}]
@@ -238,8 +238,8 @@ __global__ __launch_bounds__(64 * NW) void recon_duo_kernel(const FastParams p) 
 #pragma unroll
   for (int r = 0; r < 8; r += 2) {
     float c0, s0, c1, s1;
-    sincosf((float)n32 * p.inv_freq[16 * dq + 8 * (r >> 2) + 4 * g2 + (r & 3)], &s0, &c0);
-    sincosf((float)n32 * p.inv_freq[16 * dq + 8 * ((r + 1) >> 2) + 4 * g2 + ((r + 1) & 3)], &s1, &c1);
+    __sincosf((float)n32 * p.inv_freq[16 * dq + 8 * (r >> 2) + 4 * g2 + (r & 3)], &s0, &c0);
+    __sincosf((float)n32 * p.inv_freq[16 * dq + 8 * ((r + 1) >> 2) + 4 * g2 + ((r + 1) & 3)], &s1, &c1);
     ch[r >> 1] = rot2{(_Float16)c0, (_Float16)c1};
     sh[r >> 1] = rot2{(_Float16)s0, (_Float16)s1};
   }

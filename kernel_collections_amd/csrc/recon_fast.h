@@ -1,4 +1,4 @@
-// Interface between the recon stage-1 dispatcher and its MFMA-bound fast path (recon_fast.hip).
+// Interface between the recon stage-1 dispatcher and its MFMA-bound fast paths (recon_fast_*.hip, recon_duo_*.hip).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -17,15 +17,25 @@ struct FastParams {
   const void* vA; int64_t sVb, sVl;             // separate value basis (recon_duo kernels only)
 };
 
-int launch_recon_fast(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
-                      hipStream_t st);
+// The 4-wave kernel (recon_fast_impl.h), one translation unit per key rank: scores only, or the key basis reused as the
+// value basis.
+int launch_recon_fast_512(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
+                          hipStream_t st);
+int launch_recon_fast_384(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
+                          hipStream_t st);
+int launch_recon_fast_256(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
+                          hipStream_t st);
+inline int launch_recon_fast(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
+                             int rank, hipStream_t st) {
+  return rank == 512   ? launch_recon_fast_512(p, kB, sBb, sBh, sBr, batch, dtype, st)
+         : rank == 384 ? launch_recon_fast_384(p, kB, sBb, sBh, sBr, batch, dtype, st)
+                       : launch_recon_fast_256(p, kB, sBb, sBh, sBr, batch, dtype, st);
+}
 
-// The 8-wave kernels (recon_duo_impl.h) for key ranks 256 / 384 / 512 with scores only (mode 0), the key basis reused as
-// the value basis (mode 1) or a separate value basis of rank rv (mode 2).  Each translation unit serves the shapes it
-// instantiates and returns DUO_NOT_MINE for the others.
+// The 8-wave kernels (recon_duo_impl.h) for key ranks 256 / 384 / 512 with a separate value basis of rank rv (mode 2; the
+// kernel template also has a scores-only mode 0 and a shared-basis mode 1, which the 4-wave kernel above now serves).  Each
+// translation unit serves the shapes it instantiates and returns DUO_NOT_MINE for the others.
 constexpr int DUO_NOT_MINE = -1000;
-int launch_recon_duo_a(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
-                       int mode, int rk, int rv, hipStream_t st);
 int launch_recon_duo_b(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
                        int mode, int rk, int rv, hipStream_t st);
 int launch_recon_duo_c(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,

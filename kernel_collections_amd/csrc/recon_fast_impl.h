@@ -1,9 +1,10 @@
-// Fast path of the fused reconstruct + RoPE + softmax + P.A stage 1 (rank 512, head_dim 128, the
-// token basis shared by K and V): the MFMA-bound headline kernel.
+// Fast path of the fused reconstruct + RoPE + softmax + P.A stage 1 (rank RK = 512 / 384 / 256, head_dim 128, the
+// token basis shared by K and V): the MFMA-bound headline kernel.  Included by one translation unit per rank.
+// (Figures in the comments below are those of rank 512: 16 k-steps per wave, split 6 / 5 / 5 over the three parts.)
 //
 // Work split.  One workgroup = one (batch, kv head, split); its 4 wavefronts form a 2 x 2 grid over
-// (rank half kq, feature half dq): wave (kq, dq) keeps B[kh][256 kq .. +256][{32 dq .. +32} u {64 + 32 dq .. +32}]
-// stationary in 128 accumulation registers (both members of every rotate-half pair) and multiplies it, on
+// (rank half kq, feature half dq): wave (kq, dq) keeps B[kh][RK/2 kq .. +RK/2][{32 dq .. +32} u {64 + 32 dq .. +32}]
+// stationary in RK/4 accumulation registers (both members of every rotate-half pair) and multiplies it, on
 // v_mfma_f32_32x32x16, with its rank half of the 32-token tile.  Every element of the tile is therefore read
 // from LDS by two waves, not four - LDS read bandwidth (128 B/clk/CU), not MFMA, bounds a 4-way feature split.
 // RoPE, the rounding to the operand type and the q-dot are all linear in K, so each wave rotates and dots its
@@ -30,11 +31,13 @@
 // Tiles stream through a 4-slot LDS ring filled by direct-to-LDS loads issued three tiles ahead.  Those loads
 // are inline asm so that the compiler's wait-count pass does not serialise them against every LDS read;
 // completion is tracked by hand (s_waitcnt vmcnt(8): the 8 loads of the next tile but one may still be in flight).
+#pragma once
 #include "xkv_common.h"
 #include "recon_fast.h"
 #include <type_traits>
 
 namespace xkv {
+namespace fast {
 
 typedef short s16x4f __attribute__((ext_vector_type(4)));
 typedef short s16x8f __attribute__((ext_vector_type(8)));
@@ -42,9 +45,34 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int FT = 32;              // tokens per tile
-constexpr int FROW = 1040;          // LDS bytes per tile row (1024 + 16 pad: 16 rows hit 16 distinct bank groups)
-constexpr int FTILE = FT * FROW;    // 33280
 constexpr int FRING = 4;
+// Per rank: LDS tile geometry and the split of a wave's NKS k-steps (16 ranks each) over the three parts of an iteration.
+template <int RK> struct FastShape {
+  static_assert(RK == 512 || RK == 384 || RK == 256, "rank");
+  static constexpr int FROW = RK * 2 + 16;     // LDS bytes per tile row (16 pad: 16 rows hit 16 distinct bank groups)
+  static constexpr int FTILE = FT * FROW;
+  static constexpr int NKS = RK / 32;
+  static constexpr int P1 = RK == 512 ? 6 : RK == 384 ? 4 : 2;
+  static constexpr int P2 = RK == 512 ? 5 : RK == 384 ? 4 : 3;
+  static constexpr int P3 = NKS - P1 - P2;     // 5 / 4 / 3
+  static constexpr int NMB = RK / 64;          // 16-feature blocks of the RK / 4 latent features a wave owns in P.A
+  static_assert(3 * FROW < 4096, "instruction offset field");
+  // part 1, group o (0..3): reconstruction MFMA m (0 .. 2 P1 - 1) and the read of fragment P1 + j (j < P2)
+  static constexpr int p1_group_of_mfma(int m) { return m * 2 / P1; }
+  static constexpr int p1_group_of_read(int j) { return j < 3 ? j : 3; }
+  // part 2, group g (0..3): k-step P1 + s (s < P2), the read of fragment P1 + P2 + j (j < P3), transposed read pair mb
+  static constexpr int p2_group_of_step(int s) { return P2 == 5 ? (s < 3 ? s : s - 1) : s * 4 / P2; }
+  static constexpr int p2_group_of_read(int j) { return P3 == 5 ? (j < 1 ? 0 : j < 3 ? 1 : j - 1) : j * 4 / P3; }
+  static constexpr int p2_group_of_tr(int mb) { return mb < (NMB + 2) / 4 ? 1 : mb < 2 * ((NMB + 2) / 4) ? 2 : 3; }
+  // part 3, group u (0..4): the k-step (the last P3 groups hold one each), P.A block mb, the read of fragment j (j < P1) of
+  // the next tile, and the tile loads issued in the group (8 per tile)
+  static constexpr int p3_step(int u) { return u >= 5 - P3 ? P1 + P2 + u - (5 - P3) : -1; }
+  static constexpr int p3_group_of_pv(int mb) { return 1 + mb * 4 / NMB; }
+  static constexpr int p3_group_of_read(int j) { return j < 4 ? j : 4; }
+  static constexpr int p3_loads(int u) { return P3 == 5 ? (u == 0 || u == 4 ? 1 : 2) : (u == 0 ? 0 : 2); }
+  static constexpr int p3_first_load(int u) { return P3 == 5 ? (u == 0 ? 0 : 2 * u - 1) : 2 * u - 2; }
+  static constexpr size_t SHM = (size_t)FRING * FTILE + 4 * 8 * (FT + 4) * 4 + 2 * 8 * 128 * 2 + 16 * (FT + 8) * 2 + 16 * 4 + 16 * 4 + 128 * 2;
+};
 constexpr int FSP_ROW = FT + 4;     // partial-score row stride (floats)
 constexpr int FP_ROW = FT + 8;      // P row stride (elements)
 // The softmax reference only moves when a tile maximum exceeds it by this much.  P = exp(s - reference) is stored in the
@@ -71,20 +99,21 @@ __device__ __forceinline__ void async_row_off(const void* base_m128, unsigned vo
 template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
 // ---------------------------------------------------------------------------------------------------------------
-// kB [hkv][512][128] (strided) -> Bp [hkv][wave 4][ks 16][blk 2][lane 64][8]: the 16-byte packet lane l of wave
-// (kq, dq) feeds to MFMA (ks, blk) as the A operand: B[256 kq + 16 ks + 8 (l / 32) + e][64 blk + 32 dq + l % 32].
+// kB [hkv][RK][128] (strided) -> Bp [hkv][wave 4][ks RK/32][blk 2][lane 64][8]: the 16-byte packet lane l of wave
+// (kq, dq) feeds to MFMA (ks, blk) as the A operand: B[RK/2 kq + 16 ks + 8 (l / 32) + e][64 blk + 32 dq + l % 32].
 // ---------------------------------------------------------------------------------------------------------------
-template <typename T>
+template <typename T, int RK>
 __global__ __launch_bounds__(256) void pack_b_kernel(const T* __restrict__ kB, T* __restrict__ Bp, int64_t sBb, int64_t sBh,
                                                       int64_t sBr, int hkv) {
   const int kh = blockIdx.x, b = blockIdx.y;
   const T* Bh = kB + b * sBb + kh * sBh;
-  T* out = Bp + ((int64_t)b * hkv + kh) * (512 * 128);
-  for (int idx = blockIdx.z * 256 + threadIdx.x; idx < 4 * 16 * 2 * 64; idx += 256 * gridDim.z) {
-    const int l = idx & 63, blk = (idx >> 6) & 1, ks = (idx >> 7) & 15, w = idx >> 11;
+  constexpr int NKS = RK / 32;
+  T* out = Bp + ((int64_t)b * hkv + kh) * (RK * 128);
+  for (int idx = blockIdx.z * 256 + threadIdx.x; idx < 4 * NKS * 2 * 64; idx += 256 * gridDim.z) {
+    const int l = idx & 63, blk = (idx >> 6) & 1, ks = (idx >> 7) % NKS, w = idx / (128 * NKS);
     const int kq = w >> 1, dq = w & 1;
     const int col = 64 * blk + 32 * dq + (l & 31);
-    const int row0 = 256 * kq + 16 * ks + 8 * (l >> 5);
+    const int row0 = (RK / 2) * kq + 16 * ks + 8 * (l >> 5);
     typename Elem<T>::vec8 v;
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = Bh[(int64_t)(row0 + e) * sBr + col];
@@ -97,9 +126,11 @@ template <int V> using IC = std::integral_constant<int, V>;
 #define XKV_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)   // 0x8 MFMA, 0x2 VALU, 0x100 LDS read, 0x200 LDS write
 
 // SCORES: write the scaled scores (the qAB-with-RoPE form) instead of running softmax and P.A
-template <typename T, bool SCORES>
+template <typename T, bool SCORES, int RK>
 __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   typedef typename Elem<T>::vec8 vec8;
+  typedef FastShape<RK> S;
+  constexpr int FROW = S::FROW, FTILE = S::FTILE, NKS = S::NKS, P1 = S::P1, P2 = S::P2, P3 = S::P3, NMB = S::NMB;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -133,7 +164,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   if (tid < 16) alpha_lds[tid] = 1.f;
   if (tid < 128) qzero[tid] = from_f32<sc_t>(0.f);
 
-  // ---- async tile loads: wave w brings rows 8w .. 8w+7, one 1 KiB row per instruction ------------------------------
+  // ---- async tile loads: wave w brings rows 8w .. 8w+7, one row (RK * 2 bytes: lanes 0 .. RK/8 - 1) per instruction -----
   // Scalar row pointers advance by adds only; the clamped form is needed only where a tile crosses the split end.
   const unsigned char* Ab = reinterpret_cast<const unsigned char*>(p.kA) + b * p.sAb * 2;
   const int64_t row_bytes = p.sAl * 2;
@@ -146,13 +177,17 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   auto issue_one = [&](int t, auto r_c, auto full_c) {
     constexpr int R = decltype(r_c)::value;
     const int tok0 = start + t * FT + wave * 8;
+    const bool live = RK == 512 || lane < RK / 8;   // scalar addresses are formed outside this lane predicate
     if (decltype(full_c)::value) {
       const unsigned dst = ring_lds + (unsigned)(t & (FRING - 1)) * FTILE + (unsigned)(wave * 8 + (R & ~3)) * FROW;
-      async_row_off<(R & 3) * FROW>(Ab + (int64_t)(tok0 + (R & ~3)) * row_bytes - 128, voff4[R & 3], dst);
+      const unsigned char* base = Ab + (int64_t)(tok0 + (R & ~3)) * row_bytes - 128;
+      if (live) async_row_off<(R & 3) * FROW>(base, voff4[R & 3], dst);
     } else {
       int tok = tok0 + R;
       tok = tok < last ? tok : last;   // rows past the split end are masked in the softmax; keep the read in bounds
-      async_row16(Ab + (int64_t)tok * row_bytes, lane_off, ring_lds + (unsigned)(t & (FRING - 1)) * FTILE + (unsigned)(wave * 8 + R) * FROW);
+      const unsigned char* rowp = Ab + (int64_t)tok * row_bytes;
+      const unsigned dst = ring_lds + (unsigned)(t & (FRING - 1)) * FTILE + (unsigned)(wave * 8 + R) * FROW;
+      if (live) async_row16(rowp, lane_off, dst);
     }
   };
   auto issue_tile = [&](int t) {
@@ -163,12 +198,12 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   issue_tile(1);
   issue_tile(2);
 
-  // ---- stationary B operands: 16 k-steps x 2 feature blocks, kept in accumulation registers ---------------------------
-  vec8 breg[16][2];
+  // ---- stationary B operands: NKS k-steps x 2 feature blocks, kept in accumulation registers --------------------------
+  vec8 breg[NKS][2];
   {
-    const T* bp = reinterpret_cast<const T*>(p.Bp) + b * p.sBpb + (int64_t)kh * (512 * 128) + ((int64_t)wave * 2048 + lane) * 8;
+    const T* bp = reinterpret_cast<const T*>(p.Bp) + b * p.sBpb + (int64_t)kh * (RK * 128) + ((int64_t)wave * (128 * NKS) + lane) * 8;
 #pragma unroll
-    for (int ks = 0; ks < 16; ++ks)
+    for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk) breg[ks][blk] = ld16<vec8>(bp + (ks * 2 + blk) * 512);
   }
@@ -182,8 +217,8 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
 #pragma unroll
     for (int r = 0; r < 16; r += 2) {
       float c0, s0, c1, s1;
-      sincosf((float)(n32 + 32 * h) * p.inv_freq[32 * dq + 8 * (r >> 2) + 4 * g2 + (r & 3)], &s0, &c0);
-      sincosf((float)(n32 + 32 * h) * p.inv_freq[32 * dq + 8 * ((r + 1) >> 2) + 4 * g2 + ((r + 1) & 3)], &s1, &c1);
+      __sincosf((float)(n32 + 32 * h) * p.inv_freq[32 * dq + 8 * (r >> 2) + 4 * g2 + (r & 3)], &s0, &c0);
+      __sincosf((float)(n32 + 32 * h) * p.inv_freq[32 * dq + 8 * ((r + 1) >> 2) + 4 * g2 + ((r + 1) & 3)], &s1, &c1);
       ch[h][r >> 1] = rot2{(_Float16)c0, (_Float16)c1};
       sh[h][r >> 1] = rot2{(_Float16)s0, (_Float16)s1};
     }
@@ -290,24 +325,25 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   const int qpar = q_live ? 8 * 128 : 0;   // q^ is double-buffered by tile parity, the zeros are not
 
   // ---- accumulators and loop-carried operand registers ---------------------------------------------------------------------
-  f32x4 acc[8];          // P.A: wave w owns latent features 128 w .. +128
+  f32x4 acc[NMB];        // P.A: wave w owns latent features RK/4 w .. + RK/4
 #pragma unroll
-  for (int mb = 0; mb < 8; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int mb = 0; mb < NMB; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
   f32x16 ka[2][2];       // two sets of partial key accumulators [set][low | partner feature block]
-  vec8 at[16];           // this wave's 16 rank chunks of the tile being reconstructed (read one part ahead of their use)
+  vec8 at[NKS];          // this wave's rank chunks of the tile being reconstructed (read one part ahead of their use)
   sc_vec8 qop[4];        // q^ operands of the tile being rotated
 
   auto tile_frag = [&](int t, int ks) -> vec8 {
-    return ld16<vec8>(ring + (t & (FRING - 1)) * FTILE + n32 * FROW + (256 * kq + 8 * g2) * 2 + ks * 32);
+    return ld16<vec8>(ring + (t & (FRING - 1)) * FTILE + n32 * FROW + ((RK / 2) * kq + 8 * g2) * 2 + ks * 32);
   };
 
   // One pipeline iteration.  PAR: accumulator set written by the reconstruction of tile i; tile i-1 lives in set PAR^1.
   // Interval structure (two barriers per iteration):
-  //   part 1 [after B_c of i-1]  R(i) k-steps 0..5   ||  rotate tile i-1, q-dot, publish partial scores
+  //   part 1 [after B_c of i-1]  R(i) k-steps 0..P1-1       ||  rotate tile i-1, q-dot, publish partial scores
   //   B_b
-  //   part 2                     R(i) k-steps 6..10  ||  softmax of tile i-1; wait for tile i+1
+  //   part 2                     R(i) k-steps P1..P1+P2-1   ||  softmax of tile i-1; wait for tile i+1
   //   B_c
-  //   part 3                     R(i) k-steps 11..15 ||  acc += V^T P^T for tile i-1; issue tile i+3; write q^(i+1)
+  //   part 3                     R(i) the last P3 k-steps   ||  acc += V^T P^T for tile i-1; issue tile i+3; write q^(i+1)
+  // Which group of a part holds which MFMA, LDS read and tile load: FastShape.
   // Every LDS operand is read one part before the MFMAs that consume it.  FULL: tile i+3 lies wholly inside the split.
   auto iteration = [&](int i, auto par_c, auto do_r_c, auto do_prev_c, auto full_c) {
     constexpr int PAR = decltype(par_c)::value;
@@ -317,7 +353,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     const f32x16& j0 = ka[PAR ^ 1][0];
     const f32x16& j1 = ka[PAR ^ 1][1];
 #pragma unroll
-    for (int ks = 0; ks < 16; ++ks) {
+    for (int ks = 0; ks < NKS; ++ks) {
       asm volatile("" : "+a"(breg[ks][0]));
       asm volatile("" : "+a"(breg[ks][1]));
     }
@@ -330,10 +366,12 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
 #pragma unroll
       for (int o = 0; o < 4; ++o) {
         if (DO_R) {
-          at[6 + o] = tile_frag(i, 6 + o);
-          if (o == 3) at[10] = tile_frag(i, 10);
 #pragma unroll
-          for (int m = 3 * o; m < 3 * o + 3; ++m) {
+          for (int j = 0; j < P2; ++j)
+            if (S::p1_group_of_read(j) == o) at[P1 + j] = tile_frag(i, P1 + j);
+#pragma unroll
+          for (int m = 0; m < 2 * P1; ++m) {
+            if (S::p1_group_of_mfma(m) != o) continue;
             const int ks = m >> 1;
             if (ks == 0) {
               const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -363,7 +401,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
           // (c, g4), register r = score of token 16 (c / 8) + 4 g4 + r for head c % 8.
           sacc = Elem<sc_t>::mfma16(kop, qop[o], o == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : sacc);
         }
-        if (DO_R && DO_PREV) {   // three reconstruction MFMAs dealt out among the rotation's VALU work, then the q-dot
+        if (DO_R && DO_PREV && P1 == 6) {   // three reconstruction MFMAs dealt out among the rotation's VALU work, then the q-dot
           XKV_SGB(0x8, 1); XKV_SGB(0x2, 7);
           XKV_SGB(0x8, 1); XKV_SGB(0x2, 7);
           XKV_SGB(0x8, 1); XKV_SGB(0x2, 10);
@@ -376,9 +414,9 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     }
     __syncthreads();        // B_b: partial scores of tile i-1 are visible
     // ---- part 2 ----------------------------------------------------------------------------------------------------------
-    s16x4f tr[16];
+    s16x4f tr[2 * NMB];
     const unsigned char* vt =
-        ring + ((i - 1) & (FRING - 1)) * FTILE + (8 * g4 + (n16 >> 2)) * FROW + (wave * 128 + 4 * (n16 & 3)) * 2;
+        ring + ((i - 1) & (FRING - 1)) * FTILE + (8 * g4 + (n16 >> 2)) * FROW + (wave * (RK / 4) + 4 * (n16 & 3)) * 2;
     auto tr_read = [&](int mb) {
       if (SCORES) return;
       tr[2 * mb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4f*)(vt + mb * 32));
@@ -388,30 +426,32 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       k0 = Elem<T>::mfma32(breg[ks][0], at[ks], k0);
       k1 = Elem<T>::mfma32(breg[ks][1], at[ks], k1);
     };
+    auto part2_group = [&](auto g_c) {   // the LDS reads and k-steps FastShape assigns to group g of part 2
+      constexpr int g = decltype(g_c)::value;
+      if (DO_PREV) {
+#pragma unroll
+        for (int mb = 0; mb < NMB; ++mb)
+          if (S::p2_group_of_tr(mb) == g) tr_read(mb);   // every transposed read of tile i-1 precedes B_c
+      }
+      if (DO_R) {
+#pragma unroll
+        for (int j = 0; j < P3; ++j)
+          if (S::p2_group_of_read(j) == g) at[P1 + P2 + j] = tile_frag(i, P1 + P2 + j);
+#pragma unroll
+        for (int s2 = 0; s2 < P2; ++s2)
+          if (S::p2_group_of_step(s2) == g) recon_step(P1 + s2);
+      }
+    };
     if (DO_PREV) softmax_read();
-    if (DO_R) {
-      at[11] = tile_frag(i, 11);
-      recon_step(6);
-    }
+    part2_group(IC<0>());
     XKV_FENCE();
-    if (DO_PREV) { tr_read(0); tr_read(1); }
-    if (DO_R) {
-      at[12] = tile_frag(i, 12);
-      at[13] = tile_frag(i, 13);
-      recon_step(7);
-    }
+    part2_group(IC<1>());
     XKV_FENCE();
-    if (DO_PREV) { softmax_tile(i - 1); tr_read(2); tr_read(3); }
-    if (DO_R) {
-      at[14] = tile_frag(i, 14);
-      recon_step(8);
-      recon_step(9);
-    }
+    if (DO_PREV) softmax_tile(i - 1);
+    part2_group(IC<2>());
     XKV_FENCE();
-    if (DO_PREV) { tr_read(4); tr_read(5); tr_read(6); tr_read(7); }   // every transposed read of tile i-1 precedes B_c
+    part2_group(IC<3>());
     if (DO_R) {
-      at[15] = tile_frag(i, 15);
-      recon_step(10);
       wait_vmcnt<8>();      // this wave's rows of tile i+1 have landed (the 8 loads of tile i+2 may be in flight)
     } else {
       wait_vmcnt<0>();
@@ -424,7 +464,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
                             // the transposed reads of tile i-1 have returned, so its ring slot is free
     // ---- part 3 ----------------------------------------------------------------------------------------------------------
     vec8 pb;
-    vec8 at_next[6];
+    vec8 at_next[P1];
     sc_vec8 qop_next[4];
     const sc_t* qrow = qsrc + ((i >> 1) & 1) * qpar;   // q^ of the pair of tiles i (even) opens
     auto pv_step = [&](int mb) {
@@ -437,48 +477,53 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
       al = alpha_lds[n16];
       pb = ld16<vec8>(p_lds + n16 * FP_ROW + 8 * g4);
     }
-    if (DO_R) {
-      at_next[0] = tile_frag(i + 1, 0);
-      k0 = Elem<T>::mfma32(breg[11][0], at[11], k0);
-      XKV_FENCE();
-      issue_one(i + 3, IC<0>(), full_c);
-      XKV_FENCE();
-      k1 = Elem<T>::mfma32(breg[11][1], at[11], k1);
-    }
-    XKV_FENCE();
-    if (DO_PREV && !SCORES) {   // the two MFMAs above cover the LDS latency of the rescale factor this branch waits for
-      if (__builtin_amdgcn_ballot_w64(al != 1.f)) {   // rare: the softmax reference moved
-#pragma unroll
-        for (int mb = 0; mb < 8; ++mb) acc[mb] *= al;
-      }
-    }
+    // Group u of part 3: the P.A blocks, the k-step, the reads of the next tile's first fragments and of q^, and the tile
+    // loads FastShape assigns to it; every load sits behind an MFMA of its own where the group has one.
     auto grp = [&](auto u_c) {
       constexpr int u = decltype(u_c)::value;
-      if (DO_PREV) {
-        pv_step(2 * u - 2);
-        pv_step(2 * u - 1);
+      constexpr int ks = S::p3_step(u), nl = S::p3_loads(u), l0 = S::p3_first_load(u);
+      if (DO_PREV && u >= 1) {
+#pragma unroll
+        for (int mb = 0; mb < NMB; ++mb)
+          if (S::p3_group_of_pv(mb) == u) pv_step(mb);
       }
       if (DO_R) {
-        at_next[u] = tile_frag(i + 1, u);
-        if (u == 4) at_next[5] = tile_frag(i + 1, 5);
-        if (PAR == 0) qop_next[u - 1] = ld16<sc_vec8>(qrow + (u - 1) * 32);   // an odd tile keeps its predecessor's
-        k0 = Elem<T>::mfma32(breg[11 + u][0], at[11 + u], k0);
-        XKV_FENCE();
-        issue_one(i + 3, IC<2 * u - 1>(), full_c);
-        XKV_FENCE();
-        k1 = Elem<T>::mfma32(breg[11 + u][1], at[11 + u], k1);
-        if (u < 4) {
+#pragma unroll
+        for (int j = 0; j < P1; ++j)
+          if (S::p3_group_of_read(j) == u) at_next[j] = tile_frag(i + 1, j);
+        if (u >= 1 && PAR == 0) qop_next[u >= 1 ? u - 1 : 0] = ld16<sc_vec8>(qrow + (u - 1) * 32);   // an odd tile keeps its predecessor's
+        if (ks >= 0) {
+          constexpr int kk = ks >= 0 ? ks : 0;
+          k0 = Elem<T>::mfma32(breg[kk][0], at[kk], k0);
+          if (nl >= 1) {
+            XKV_FENCE();
+            issue_one(i + 3, IC<l0>(), full_c);        // into the ring slot of tile i-1, whose readers are done
+            XKV_FENCE();
+          }
+          k1 = Elem<T>::mfma32(breg[kk][1], at[kk], k1);
+          if (nl >= 2) {
+            XKV_FENCE();
+            issue_one(i + 3, IC<l0 + 1>(), full_c);
+          }
+        } else if (nl > 0) {
           XKV_FENCE();
-          issue_one(i + 3, IC<2 * u>(), full_c);
+          issue_one(i + 3, IC<l0>(), full_c);
+          if (nl >= 2) issue_one(i + 3, IC<(nl >= 2 ? l0 + 1 : l0)>(), full_c);
         }
         if (u == 4 && PAR == 1) write_qhat(i + 1);   // buffer ((i+1)/2)&1 was last read in part 3 of iteration i-3
       }
       XKV_FENCE();
+      if (u == 0 && DO_PREV && !SCORES) {   // the MFMAs above cover the LDS latency of the rescale factor this branch waits for
+        if (__builtin_amdgcn_ballot_w64(al != 1.f)) {   // rare: the softmax reference moved
+#pragma unroll
+          for (int mb = 0; mb < NMB; ++mb) acc[mb] *= al;
+        }
+      }
     };
-    grp(IC<1>()); grp(IC<2>()); grp(IC<3>()); grp(IC<4>());
+    grp(IC<0>()); grp(IC<1>()); grp(IC<2>()); grp(IC<3>()); grp(IC<4>());
     if (DO_R) {
 #pragma unroll
-      for (int ks = 0; ks < 6; ++ks) at[ks] = at_next[ks];
+      for (int ks = 0; ks < P1; ++ks) at[ks] = at_next[ks];
 #pragma unroll
       for (int o = 0; o < 4; ++o)
         if (PAR == 0) qop[o] = qop_next[o];
@@ -489,7 +534,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   wait_vmcnt<0>();          // tiles 0..2 and the B operands
   __syncthreads();
 #pragma unroll
-  for (int ks = 0; ks < 6; ++ks) at[ks] = tile_frag(0, ks);
+  for (int ks = 0; ks < P1; ++ks) at[ks] = tile_frag(0, ks);
   const int nfull = (end - start) / FT;
   iteration(0, IC<0>(), IC<1>(), IC<0>(), IC<0>());
   int i = 1;
@@ -519,32 +564,33 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
     const float m = ml_lds[2 * n16], l = ml_lds[2 * n16 + 1];
     const float inv = 1.f / l;
     const int64_t ph = ((int64_t)b * p.hq + h0 + n16) * p.max_splits + split;
-    float* dst = p.partial + ph * 512 + wave * 128 + 4 * g4;
+    float* dst = p.partial + ph * RK + wave * (RK / 4) + 4 * g4;
 #pragma unroll
-    for (int mb = 0; mb < 8; ++mb) *reinterpret_cast<f32x4*>(dst + mb * 16) = acc[mb] * inv;
+    for (int mb = 0; mb < NMB; ++mb) *reinterpret_cast<f32x4*>(dst + mb * 16) = acc[mb] * inv;
     if (wave == 0 && g4 == 0) p.lse[ph] = m + __logf(l);
   }
 }
 
-constexpr size_t FAST_SHM = (size_t)FRING * FTILE + 4 * 8 * FSP_ROW * 4 + 2 * 8 * 128 * 2 + 16 * FP_ROW * 2 + 16 * 4 + 16 * 4 + 128 * 2;
-
-template <typename T>
+template <typename T, int RK>
 int launch_recon_fast_t(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, hipStream_t st) {
+  typedef FastShape<RK> S;
   const int nb = sBb == 0 ? 1 : batch;   // one packed copy when the factor is shared by the batch
-  pack_b_kernel<T><<<dim3(p.hkv, nb, 32), dim3(256), 0, st>>>((const T*)kB, (T*)p.Bp, sBb, sBh, sBr, p.hkv);
-  auto kern = p.scores ? recon_fast_kernel<T, true> : recon_fast_kernel<T, false>;
+  pack_b_kernel<T, RK><<<dim3(p.hkv, nb, 32), dim3(256), 0, st>>>((const T*)kB, (T*)p.Bp, sBb, sBh, sBr, p.hkv);
+  auto kern = p.scores ? recon_fast_kernel<T, true, RK> : recon_fast_kernel<T, false, RK>;
   static DynLds lds[2];
-  hipError_t e = ensure_dynamic_lds(lds[p.scores ? 1 : 0], reinterpret_cast<const void*>(kern), (int)FAST_SHM);
+  hipError_t e = ensure_dynamic_lds(lds[p.scores ? 1 : 0], reinterpret_cast<const void*>(kern), (int)S::SHM);
   if (e != hipSuccess) return (int)e;
   const int total = batch * p.hkv * p.max_splits;
-  kern<<<dim3(xcd_grid(total, p.hkv)), dim3(256), FAST_SHM, st>>>(p);
+  kern<<<dim3(xcd_grid(total, p.hkv)), dim3(256), S::SHM, st>>>(p);
   return launch_status();
 }
 
-int launch_recon_fast(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
-                      hipStream_t st) {
-  return dtype == XKV_BF16 ? launch_recon_fast_t<__bf16>(p, kB, sBb, sBh, sBr, batch, st)
-                           : launch_recon_fast_t<_Float16>(p, kB, sBb, sBh, sBr, batch, st);
+template <int RK>
+int launch_recon_fast_rank(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
+                           hipStream_t st) {
+  return dtype == XKV_BF16 ? launch_recon_fast_t<__bf16, RK>(p, kB, sBb, sBh, sBr, batch, st)
+                           : launch_recon_fast_t<_Float16, RK>(p, kB, sBb, sBh, sBr, batch, st);
 }
 
+}  // namespace fast
 }  // namespace xkv

@@ -401,24 +401,11 @@ extern "C" int xkv_recon_stage1(const void* q_pe, xkv_kv_operand kA, const void*
   const bool vshared = !so && vA.ptr == kA.ptr && vA.stride_b == kA.stride_b && vA.stride_l == kA.stride_l &&
                        vA.dim == kA.dim;
   hipStream_t st = (hipStream_t)stream;
-  // MFMA-bound fast path: rank 512, scores only or a basis shared by K and V, computed RoPE angles, at most 8 query heads
+  // MFMA-bound fast path: rank 512 / 384 / 256, scores only or a basis shared by K and V, computed RoPE angles, at most 8 query heads
   // per kv head
   const int64_t need = xkv_recon_workspace_bytes(batch, hkv, rank, sBb);
-  if ((so || vshared) && rope && !sin_cos && rank == 512 && hq / hkv <= 8 && workspace && need > 0 &&
+  if ((so || vshared) && rope && !sin_cos && (rank == 512 || rank == 384 || rank == 256) && hq / hkv <= 8 && workspace && need > 0 &&
       workspace_bytes >= need && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
-    FastParams f;
-    f.q = q_pe; f.kA = kA.ptr; f.Bp = workspace;
-    f.sAb = kA.stride_b; f.sAl = kA.stride_l; f.sBpb = sBb == 0 ? 0 : (int64_t)hkv * 512 * 128;
-    f.partial = partial; f.lse = lse; f.scores = scores_out; f.scores_dtype = scores_dtype;
-    f.num_splits = num_kv_splits; f.kv_lens = kv_lens;
-    f.hq = hq; f.hkv = hkv; f.kv_len = kv_len; f.max_splits = max_splits; f.total_wg = batch * hkv * max_splits;
-    f.sm_scale = sm_scale; f.inv_freq = inv_freq; f.pos_offset = pos_offset;
-    return launch_recon_fast(f, kB, sBb, sBh, sBr, batch, dtype, st);
-  }
-  // 8-wave kernels: the other ranks, and a value basis of its own
-  if (rope && !sin_cos && hq / hkv <= 8 && workspace && need > 0 && workspace_bytes >= need &&
-      (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 && (int64_t)kA.stride_l * 2 * 3 < ((int64_t)1 << 31) &&
-      (so || vshared || (int64_t)vA.stride_l * 2 * 3 < ((int64_t)1 << 31))) {
     FastParams f;
     f.q = q_pe; f.kA = kA.ptr; f.Bp = workspace;
     f.sAb = kA.stride_b; f.sAl = kA.stride_l; f.sBpb = sBb == 0 ? 0 : (int64_t)hkv * rank * 128;
@@ -426,11 +413,22 @@ extern "C" int xkv_recon_stage1(const void* q_pe, xkv_kv_operand kA, const void*
     f.num_splits = num_kv_splits; f.kv_lens = kv_lens;
     f.hq = hq; f.hkv = hkv; f.kv_len = kv_len; f.max_splits = max_splits; f.total_wg = batch * hkv * max_splits;
     f.sm_scale = sm_scale; f.inv_freq = inv_freq; f.pos_offset = pos_offset;
+    return launch_recon_fast(f, kB, sBb, sBh, sBr, batch, dtype, rank, st);
+  }
+  // 8-wave kernels: a value basis of its own beside key ranks 256 / 384 / 512
+  if (!so && !vshared && rope && !sin_cos && hq / hkv <= 8 && workspace && need > 0 && workspace_bytes >= need &&
+      (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 && (int64_t)kA.stride_l * 2 * 3 < ((int64_t)1 << 31) &&
+      (int64_t)vA.stride_l * 2 * 3 < ((int64_t)1 << 31)) {
+    FastParams f;
+    f.q = q_pe; f.kA = kA.ptr; f.Bp = workspace;
+    f.sAb = kA.stride_b; f.sAl = kA.stride_l; f.sBpb = sBb == 0 ? 0 : (int64_t)hkv * rank * 128;
+    f.partial = partial; f.lse = lse; f.scores = nullptr; f.scores_dtype = scores_dtype;
+    f.num_splits = num_kv_splits; f.kv_lens = kv_lens;
+    f.hq = hq; f.hkv = hkv; f.kv_len = kv_len; f.max_splits = max_splits; f.total_wg = batch * hkv * max_splits;
+    f.sm_scale = sm_scale; f.inv_freq = inv_freq; f.pos_offset = pos_offset;
     f.vA = vA.ptr; f.sVb = vA.stride_b; f.sVl = vA.stride_l;
-    const int mode = so ? 0 : vshared ? 1 : 2, rv = so ? rank : vA.dim;
-    int rc = launch_recon_duo_a(f, kB, sBb, sBh, sBr, batch, dtype, mode, rank, rv, st);
-    if (rc == DUO_NOT_MINE) rc = launch_recon_duo_b(f, kB, sBb, sBh, sBr, batch, dtype, mode, rank, rv, st);
-    if (rc == DUO_NOT_MINE) rc = launch_recon_duo_c(f, kB, sBb, sBh, sBr, batch, dtype, mode, rank, rv, st);
+    int rc = launch_recon_duo_b(f, kB, sBb, sBh, sBr, batch, dtype, 2, rank, vA.dim, st);
+    if (rc == DUO_NOT_MINE) rc = launch_recon_duo_c(f, kB, sBb, sBh, sBr, batch, dtype, 2, rank, vA.dim, st);
     if (rc != DUO_NOT_MINE) return rc;
   }
   return dtype == XKV_BF16 ? dispatch_recon<__bf16>(p, batch, vshared, st) : dispatch_recon<_Float16>(p, batch, vshared, st);

@@ -70,7 +70,11 @@ def decode_k_only(q, k_A, k_B, v_buffer, o, num_kv_splits, max_kv_splits, sm_sca
 
 
 # key ranks at which fused RoPE decode with a value basis of its own runs as two passes (scores, then softmax + P.v_A)
-TWO_PASS_KEY_RANKS = (512, 384)   # at rank 256 the two forms tie
+# A value basis of its own runs as two passes (scores, then softmax + P.v_A) at these key ranks once the call scans at
+# least TWO_PASS_MIN_TOKENS tokens (batch x kv_len); below, the extra launches cost more than the second row stream of
+# the fused 8-wave kernel (measured crossover: 32768 tokens at every rank).
+TWO_PASS_KEY_RANKS = (512, 384, 256)
+TWO_PASS_MIN_TOKENS = 49152
 
 
 def decode_rope(q_pe, k_A, k_B, v_A, v_B, o, num_kv_splits, max_kv_splits, sm_scale, theta, sin_cos,
@@ -98,7 +102,8 @@ def decode_rope(q_pe, k_A, k_B, v_A, v_B, o, num_kv_splits, max_kv_splits, sm_sc
         if sin_cos.dtype != q_pe.dtype or sin_cos.stride(-1) != 1:
             sin_cos = sin_cos.to(q_pe.dtype).contiguous()
     same_basis = (v_A.data_ptr() == k_A.data_ptr() and v_A.shape == k_A.shape and v_A.stride() == k_A.stride())
-    if (not same_basis and k_A.shape[-1] in TWO_PASS_KEY_RANKS and sin_cos is None and hq // hkv <= 8 and hq <= 32
+    if (not same_basis and k_A.shape[-1] in TWO_PASS_KEY_RANKS and batch * kv_len >= TWO_PASS_MIN_TOKENS
+            and sin_cos is None and hq // hkv <= 8 and hq <= 32
             and rank_v in (256, 384, 512) and kv_len % 4 == 0 and ops.USE_RECON_WORKSPACE):
         # A value basis of its own: two passes.  The scores-only form of the reconstruction kernel runs at the rate of the
         # shared-basis fused kernel (one row stream, no P.A); softmax and P.v_A then stream v_A once for all heads at HBM

@@ -215,11 +215,16 @@ def test_fused_rope(dev, dtype, b, hq, hkv, L, rk, rv, S, shared):
     (1, 24, 8, 256, 512, False, [1500], 7, 0),             # the last splits are dead
     (2, 32, 8, 384, 384, True, [900, 1200], 4, 0),
     (2, 16, 4, 256, 256, True, [33, 4000], 6, 131072 - 4000)])
-@pytest.mark.parametrize("two_pass_ranks", [(), (512, 384), (512, 384, 256)], ids=["fused", "two_pass_default", "two_pass_all"])
-def test_fused_rope_wide_kernels(dev, dtype, b, hq, hkv, rk, rv, shared, lens, S, off, two_pass_ranks, monkeypatch):
-    # a value basis of its own runs either fused (one kernel, two row streams) or as two passes (scores, then softmax + P.v_A)
+@pytest.mark.parametrize("form", ["fused", "two_pass", "as_shipped"])
+def test_fused_rope_wide_kernels(dev, dtype, b, hq, hkv, rk, rv, shared, lens, S, off, form, monkeypatch):
+    # a value basis of its own runs either fused (one kernel, two row streams) or as two passes (scores, then softmax + P.v_A);
+    # as shipped the choice follows the key rank and the number of tokens scanned: here both forms are forced in turn
     from kernel_collections_amd.flash_recontruction.fused_attention import _fused
-    monkeypatch.setattr(_fused, "TWO_PASS_KEY_RANKS", two_pass_ranks)
+    if form == "fused":
+        monkeypatch.setattr(_fused, "TWO_PASS_KEY_RANKS", ())
+    elif form == "two_pass":
+        monkeypatch.setattr(_fused, "TWO_PASS_KEY_RANKS", (512, 384, 256))
+        monkeypatch.setattr(_fused, "TWO_PASS_MIN_TOKENS", 0)
     d, theta = 128, 5e5
     L = max(lens)
     q = gen((b, hq, d), std=0.4, dtype=dtype, seed=21)
