@@ -108,7 +108,8 @@ def test_qab_nope_shared_factor_stride0_and_row_strides(dev):
 @pytest.mark.parametrize("dtype", [BF, FP])
 @pytest.mark.parametrize("b,hq,hkv,L,r,theta", [(2, 32, 8, 1000, 512, 5e5), (1, 8, 2, 77, 256, 1e7),
                                                 (1, 16, 1, 2085, 384, 1e4), (2, 4, 4, 40, 192, 1e7),
-                                                (2, 8, 2, 300, 384, 5e5)])   # 8-wave kernel, scores mode
+                                                (2, 8, 2, 300, 384, 5e5),    # 4-wave kernel at rank 384, scores mode
+                                                (1, 16, 2, 1500, 256, 1e7)])  # ... at rank 256, 8 heads per kv head
 def test_qab_rope(dev, dtype, b, hq, hkv, L, r, theta):
     d = 128
     q, A, B = gen((b, hq, 1, d), std=0.5, dtype=dtype, seed=1), gen((b, L, r), dtype=dtype, seed=2), \
@@ -208,13 +209,15 @@ def test_fused_rope(dev, dtype, b, hq, hkv, L, rk, rv, S, shared):
 
 @pytest.mark.parametrize("dtype", [BF, FP])
 @pytest.mark.parametrize("b,hq,hkv,rk,rv,shared,lens,S,off", [
-    (2, 32, 8, 512, 512, False, [1000, 333], 4, 0),        # every shape the 8-wave kernels are built for
+    (2, 32, 8, 512, 512, False, [1000, 333], 4, 0),        # every shape the 8-wave kernels are built for (fused form)
     (1, 16, 2, 384, 512, False, [2100], 3, 4096),          # 8 query heads per kv head
     (2, 8, 8, 384, 384, False, [17, 64], 2, 0),            # shorter than a tile / exactly two tiles; one head per kv head
     (3, 32, 8, 256, 256, False, [700, 5, 2048], 5, 100000),
     (1, 24, 8, 256, 512, False, [1500], 7, 0),             # the last splits are dead
     (2, 32, 8, 384, 384, True, [900, 1200], 4, 0),
-    (2, 16, 4, 256, 256, True, [33, 4000], 6, 131072 - 4000)])
+    (2, 16, 4, 256, 256, True, [33, 4000], 6, 131072 - 4000),
+    (1, 16, 2, 384, 384, True, [1500], 3, 0),              # the 4-wave kernel at ranks 384 / 256: 8 heads per kv head ...
+    (2, 8, 8, 256, 256, True, [100, 257], 2, 50000)])      # ... and one
 @pytest.mark.parametrize("form", ["fused", "two_pass", "as_shipped"])
 def test_fused_rope_wide_kernels(dev, dtype, b, hq, hkv, rk, rv, shared, lens, S, off, form, monkeypatch):
     # a value basis of its own runs either fused (one kernel, two row streams) or as two passes (scores, then softmax + P.v_A);

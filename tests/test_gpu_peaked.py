@@ -182,7 +182,7 @@ PATHS = {
     "recon_fast(r512 shared, positions near 128K)": ReconRope(512, 512, True, off=131072 - 1500),
     "recon_duo(r384/512)": ReconRope(384, 512, False),
     "recon_duo(r512/512)": ReconRope(512, 512, False),
-    "recon_duo(r256 shared, G 8)": ReconRope(256, 256, True, hq=16, hkv=2),
+    "recon_fast(r256 shared, G 8)": ReconRope(256, 256, True, hq=16, hkv=2),
     "recon_stage1(r192 shared)": ReconRope(192, 192, True),
     "recon_stage1(r512 table)": ReconRope(512, 512, True, table=True),
     "latent_ring(absorbed r512/512)": FusedNope(512, 512),
