@@ -109,8 +109,11 @@ def decode_rope(q_pe, k_A, k_B, v_A, v_B, o, num_kv_splits, max_kv_splits, sm_sc
         # shared-basis fused kernel (one row stream, no P.A); softmax and P.v_A then stream v_A once for all heads at HBM
         # rate.  Fused into one kernel, the second row stream costs more than the 2 x 4 bytes per score this moves.
         scores = torch.empty((batch, hq, kv_len), dtype=torch.float32, device=q_pe.device)
-        ops.recon_stage1(q3, k_A, k_B, None, None, None, scores, splits, lens, batch, hq, hkv, kv_len, S,
-                         float(sm_scale), True, inv, int(pos_offset), None)
+        # the scores do not depend on how pass 1 cuts the range: one round of workgroups per CU, two at key rank 256, whose
+        # scores-only kernel is small enough for two workgroups to share a CU
+        S1 = ops.occupancy_splits(batch, hkv, kv_len, tile=32, waves=2 if k_A.shape[-1] == 256 else 1)
+        ops.recon_stage1(q3, k_A, k_B, None, None, None, scores, ops.uniform_splits(batch, S1, q_pe.device), lens, batch, hq,
+                         hkv, kv_len, S1, float(sm_scale), True, inv, int(pos_offset), None)
         S2 = ops.latent_splits(batch, 1, kv_len, rank_v, absorbed=True)
         splits2 = ops.uniform_splits(batch, S2, q_pe.device)
         partial, lse = ops.workspaces(batch, hq, S2, rank_v, q_pe.device)
