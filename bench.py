@@ -628,7 +628,7 @@ def bench_ropedecode(args, dev):
         "ms_per_step": total_ms / args.steps, "step_us": step_q,
         "config": {"workload": "fused RoPE xKV decode, separate bases: batch 1, 32q/8kv, d128, kv_len %d, K rank %d, V rank %d, bf16"
                                % (L, rk, rv), "kv_splits": S},
-        "roofline": {"bound": "mfma", "kernel": "recon_duo_kernel (scores) + latent_ring_kernel (given scores), two passes", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": "recon_fast_kernel (scores) + latent_ring_kernel (given scores), two passes", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
                      "note": "whole call (pack, stage 1, merge) over algorithmic FLOP", "algorithmic_flop": flops,
                      "hbm_side_GBps": round(B * L * (rk + rv) * 2 / (us * 1e-6) / 1e9, 1)},
