@@ -1,6 +1,6 @@
 // Fast path of the fused reconstruct + RoPE + softmax + P.A stage 1 (rank RK = 512 / 384 / 256, head_dim 128, the
 // token basis shared by K and V): the MFMA-bound headline kernel.  Included by one translation unit per rank.
-// (Figures in the comments below are those of rank 512: 16 k-steps per wave, split 6 / 5 / 5 over the three parts.)
+// (Figures in the comments below are those of rank 512: 16 k-steps per wave, split 5 / 6 / 5 over the three parts.)
 //
 // Work split.  One workgroup = one (batch, kv head, split); its 4 wavefronts form a 2 x 2 grid over
 // (rank half kq, feature half dq): wave (kq, dq) keeps B[kh][RK/2 kq .. +RK/2][{32 dq .. +32} u {64 + 32 dq .. +32}]
@@ -19,8 +19,8 @@
 // Pipeline.  A wave issues instructions in order, so MFMA time and VALU time only overlap when independent
 // work is interleaved in its instruction stream.  Iteration i therefore runs the 16 reconstruction MFMA steps of
 // tile i (accumulating into one of two key-accumulator sets) in three parts, interleaved with what tile i-1 still
-// needs: part 1 (steps 0..5) rotates tile i-1's partial keys (the other accumulator set) in packed fp16, dots them
-// with q^ on v_mfma_f32_16x16x32 and stores the partial scores; barrier; part 2 (steps 6..10) runs the softmax of
+// needs: part 1 (steps 0..4) rotates tile i-1's partial keys (the other accumulator set) in packed fp16, dots them
+// with q^ on v_mfma_f32_16x16x32 and stores the partial scores; barrier; part 2 (steps 5..10) runs the softmax of
 // tile i-1 (one owner lane group per head: no redundant work), publishes P and the rescale factor through LDS and
 // reads tile i-1 transposed for P.A; barrier; part 3 (steps 11..15) accumulates P.A for tile i-1, each wave owning
 // 128 latent features, issues the loads of tile i+3 into the slot tile i-1 has left (one load behind each MFMA),
@@ -52,9 +52,10 @@ template <int RK> struct FastShape {
   static constexpr int FROW = RK * 2 + 16;     // LDS bytes per tile row (16 pad: 16 rows hit 16 distinct bank groups)
   static constexpr int FTILE = FT * FROW;
   static constexpr int NKS = RK / 32;
-  static constexpr int P1 = RK == 512 ? 6 : RK == 384 ? 4 : 2;
-  static constexpr int P2 = RK == 512 ? 5 : RK == 384 ? 4 : 3;
+  static constexpr int P1 = RK == 512 ? 5 : RK == 384 ? 4 : 2;
+  static constexpr int P2 = RK == 512 ? 6 : RK == 384 ? 4 : 3;   // part 2 carries the softmax chain: the longest share at rank 512
   static constexpr int P3 = NKS - P1 - P2;     // 5 / 4 / 3
+  static_assert(P3 <= 5 && P1 >= 1 && P2 >= 1, "part 3 has five groups, one k-step each");
   static constexpr int NMB = RK / 64;          // 16-feature blocks of the RK / 4 latent features a wave owns in P.A
   static_assert(3 * FROW < 4096, "instruction offset field");
   // part 1, group o (0..3): reconstruction MFMA m (0 .. 2 P1 - 1) and the read of fragment P1 + j (j < P2)
@@ -123,7 +124,6 @@ __global__ __launch_bounds__(256) void pack_b_kernel(const T* __restrict__ kB, T
 
 template <int V> using IC = std::integral_constant<int, V>;
 #define XKV_FENCE() __builtin_amdgcn_sched_barrier(0)
-#define XKV_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)   // 0x8 MFMA, 0x2 VALU, 0x100 LDS read, 0x200 LDS write
 
 // SCORES: write the scaled scores (the qAB-with-RoPE form) instead of running softmax and P.A
 template <typename T, bool SCORES, int RK>
@@ -400,12 +400,6 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
           // column c holds q^ of head c % 8 in the k-groups of token half c / 8 and zeros in the other two.  Result: lane
           // (c, g4), register r = score of token 16 (c / 8) + 4 g4 + r for head c % 8.
           sacc = Elem<sc_t>::mfma16(kop, qop[o], o == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : sacc);
-        }
-        if (DO_R && DO_PREV && P1 == 6) {   // three reconstruction MFMAs dealt out among the rotation's VALU work, then the q-dot
-          XKV_SGB(0x8, 1); XKV_SGB(0x2, 7);
-          XKV_SGB(0x8, 1); XKV_SGB(0x2, 7);
-          XKV_SGB(0x8, 1); XKV_SGB(0x2, 10);
-          XKV_SGB(0x8, 1);
         }
         XKV_FENCE();
       }
