@@ -47,14 +47,16 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 constexpr int FT = 32;              // tokens per tile
 constexpr int FRING = 4;
 // Per rank: LDS tile geometry and the split of a wave's NKS k-steps (16 ranks each) over the three parts of an iteration.
-template <int RK> struct FastShape {
+template <int RK, bool SCORES> struct FastShape {
   static_assert(RK == 512 || RK == 384 || RK == 256, "rank");
   static constexpr int FROW = RK * 2 + 16;     // LDS bytes per tile row (16 pad: 16 rows hit 16 distinct bank groups)
   static constexpr int FTILE = FT * FROW;
   static constexpr int NKS = RK / 32;
-  static constexpr int P1 = RK == 512 ? 5 : RK == 384 ? 4 : 2;
-  static constexpr int P2 = RK == 512 ? 6 : RK == 384 ? 4 : 3;   // part 2 carries the softmax chain: the longest share at rank 512
-  static constexpr int P3 = NKS - P1 - P2;     // 5 / 4 / 3
+  // measured, the best of the splits tried at each rank: 5+6+5, 5+5+2, and at rank 256 3+4+1 (fused) / 3+3+2 (scores only:
+  // the split that keeps that instantiation small enough for two workgroups per CU)
+  static constexpr int P1 = RK == 512 ? 5 : RK == 384 ? 5 : 3;
+  static constexpr int P2 = RK == 512 ? 6 : RK == 384 ? 5 : SCORES ? 3 : 4;
+  static constexpr int P3 = NKS - P1 - P2;
   static_assert(P3 <= 5 && P1 >= 1 && P2 >= 1, "part 3 has five groups, one k-step each");
   static constexpr int NMB = RK / 64;          // 16-feature blocks of the RK / 4 latent features a wave owns in P.A
   static_assert(3 * FROW < 4096, "instruction offset field");
@@ -129,7 +131,7 @@ template <int V> using IC = std::integral_constant<int, V>;
 template <typename T, bool SCORES, int RK>
 __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
   typedef typename Elem<T>::vec8 vec8;
-  typedef FastShape<RK> S;
+  typedef FastShape<RK, SCORES> S;
   constexpr int FROW = S::FROW, FTILE = S::FTILE, NKS = S::NKS, P1 = S::P1, P2 = S::P2, P3 = S::P3, NMB = S::NMB;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -567,7 +569,7 @@ __global__ __launch_bounds__(256) void recon_fast_kernel(const FastParams p) {
 
 template <typename T, int RK>
 int launch_recon_fast_t(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, hipStream_t st) {
-  typedef FastShape<RK> S;
+  typedef FastShape<RK, false> S;   // the LDS footprint does not depend on the mode
   const int nb = sBb == 0 ? 1 : batch;   // one packed copy when the factor is shared by the batch
   pack_b_kernel<T, RK><<<dim3(p.hkv, nb, 32), dim3(256), 0, st>>>((const T*)kB, (T*)p.Bp, sBb, sBh, sBr, p.hkv);
   auto kern = p.scores ? recon_fast_kernel<T, true, RK> : recon_fast_kernel<T, false, RK>;
