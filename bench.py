@@ -31,7 +31,7 @@ PEAK_BF16_TFLOPS = 2500.0
 # HBM bytes of one stage-1 launch at the default c3 shape, from two rocprofv3 --pmc runs of this file
 # (FETCH_SIZE, WRITE_SIZE; each scaled by what the counter reads for --calib-copy's 512 MiB copies).
 # A counter cannot be read from inside the timed process, so the figure is recorded here.
-C3_STAGE1_HBM_BYTES = 537278 * 1024     # recon_fast_kernel 2 x 266578.5 + 2056.0 KiB, pack_b_kernel 2 x 520.5 + 1024 KiB
+C3_STAGE1_HBM_BYTES = 537274 * 1024     # recon_fast_kernel 2 x 266578.5 + 2056.0 KiB, pack_b_kernel 2 x 518.5 + 1024 KiB
 C5_RING_HBM_BYTES = 604800 * 1024       # same method, latent_ring_kernel at the default c5 shape (2 x 298272.1 + 8256.0 KiB)
 C2_RING_HBM_BYTES = 151785 * 1024       # latent_ring_kernel, scores mode, default c2 shape (2 x 67700.4 + 16384.0 KiB)
 C4_RING_HBM_BYTES = 3022744 * 1024      # latent_ring_kernel at c4 plain with the planned split length (2 x 1509401.8 + 3940.0 KiB)
