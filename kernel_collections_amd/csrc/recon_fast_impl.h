@@ -6,15 +6,15 @@
 // (rank half kq, feature half dq): wave (kq, dq) keeps B[kh][RK/2 kq .. +RK/2][{32 dq .. +32} u {64 + 32 dq .. +32}]
 // stationary in RK/4 accumulation registers (both members of every rotate-half pair) and multiplies it, on
 // v_mfma_f32_32x32x16, with its rank half of the 32-token tile.  Every element of the tile is therefore read
-// from LDS by two waves, not four - LDS read bandwidth (128 B/clk/CU), not MFMA, bounds a 4-way feature split.
+// from LDS by two waves, not four - LDS reads, not MFMA, bound a 4-way feature split.
 // RoPE, the rounding to the operand type and the q-dot are all linear in K, so each wave rotates and dots its
 // PARTIAL key tile (partial over its rank half and its feature half) and only 4 x [G x 32] fp32 partial scores
 // are summed through LDS.
 //
-// Rotation.  R(pos) = R(tile base) R(offset in tile).  The in-tile part is a per-lane constant table (32
-// VGPRs); the base part is moved to the query: q^ = R(-base) q is recomputed per tile by the workgroup
-// (one thread per pair index, incremental rotation re-seeded with a range-reduced sincosf every 32 tiles)
-// and read back as the B operand of the q-dot MFMA.
+// Rotation.  R(pos) = R(base) R(offset).  The base is that of an even tile and is moved to the query: q^ = R(-base) q
+// is recomputed once per two tiles by the workgroup (one thread per pair index, incremental rotation re-seeded with a
+// range-reduced sincosf every 32 tiles) and read back as the B operand of the q-dot MFMA; the offset part (0..31 for
+// the even tile, 32..63 for the odd one) is two per-lane constant tables in fp16 (32 VGPRs).
 //
 // Pipeline.  A wave issues instructions in order, so MFMA time and VALU time only overlap when independent
 // work is interleaved in its instruction stream.  Iteration i therefore runs the 16 reconstruction MFMA steps of
@@ -23,8 +23,8 @@
 // with q^ on v_mfma_f32_16x16x32 and stores the partial scores; barrier; part 2 (steps 5..10) runs the softmax of
 // tile i-1 (one owner lane group per head: no redundant work), publishes P and the rescale factor through LDS and
 // reads tile i-1 transposed for P.A; barrier; part 3 (steps 11..15) accumulates P.A for tile i-1, each wave owning
-// 128 latent features, issues the loads of tile i+3 into the slot tile i-1 has left (one load behind each MFMA),
-// writes q^ for tile i+1 and prefetches the first LDS operands of tile i+1.  Two barriers per tile separate the parts.
+// RK/4 latent features, issues the loads of tile i+3 into the slot tile i-1 has left (one load behind each MFMA),
+// writes q^ for the next pair of tiles and prefetches the first LDS operands of tile i+1.  Two barriers per tile separate the parts.
 // The softmax reference only moves when a tile maximum exceeds it by 16 (8 for fp16 operands: lazy rescaling), so the
 // P.A accumulators are almost never rescaled.
 //
