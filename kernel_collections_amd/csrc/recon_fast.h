@@ -25,6 +25,13 @@ int launch_recon_fast_384(const FastParams& p, const void* kB, int64_t sBb, int6
                           hipStream_t st);
 int launch_recon_fast_256(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
                           hipStream_t st);
+// The wave-specialised 8-wave kernel (recon_spec_impl.h): the same shapes and arguments as the 4-wave kernel.
+int launch_recon_spec_512(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
+                          hipStream_t st);
+int launch_recon_spec_384(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
+                          hipStream_t st);
+int launch_recon_spec_256(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
+                          hipStream_t st);
 inline int launch_recon_fast(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
                              int rank, hipStream_t st) {
   return rank == 512   ? launch_recon_fast_512(p, kB, sBb, sBh, sBr, batch, dtype, st)
