@@ -23,7 +23,7 @@ FLAGS = [
 # pinned to accumulation registers by the source itself.
 _VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 EXTRA_FLAGS = {
-    "recon_fast_512.hip": _VGPR_FORM, "recon_fast_384.hip": _VGPR_FORM, "recon_fast_256.hip": _VGPR_FORM,
+    "recon_fast_256.hip": _VGPR_FORM,
     "recon_duo_b.hip": _VGPR_FORM, "recon_duo_c.hip": _VGPR_FORM, "recon_spec_512.hip": _VGPR_FORM, "recon_spec_384.hip": _VGPR_FORM, "recon_spec_256.hip": _VGPR_FORM,
 }
 

@@ -17,26 +17,22 @@ struct FastParams {
   const void* vA; int64_t sVb, sVl;             // separate value basis (recon_duo kernels only)
 };
 
-// The 4-wave kernel (recon_fast_impl.h), one translation unit per key rank: scores only, or the key basis reused as the
-// value basis.
-int launch_recon_fast_512(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
-                          hipStream_t st);
-int launch_recon_fast_384(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
-                          hipStream_t st);
+// The 4-wave kernel (recon_fast_impl.h): scores only, or the key basis reused as the value basis.  Instantiated at rank 256,
+// where its scores-only form fits a CU twice.
 int launch_recon_fast_256(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
                           hipStream_t st);
-// The wave-specialised 8-wave kernel (recon_spec_impl.h): the same shapes and arguments as the 4-wave kernel.
+// The wave-specialised 8-wave kernel (recon_spec_impl.h), one translation unit per key rank: the same shapes and arguments.
 int launch_recon_spec_512(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
                           hipStream_t st);
 int launch_recon_spec_384(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
                           hipStream_t st);
 int launch_recon_spec_256(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
                           hipStream_t st);
-inline int launch_recon_fast(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
+inline int launch_recon_spec(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,
                              int rank, hipStream_t st) {
-  return rank == 512   ? launch_recon_fast_512(p, kB, sBb, sBh, sBr, batch, dtype, st)
-         : rank == 384 ? launch_recon_fast_384(p, kB, sBb, sBh, sBr, batch, dtype, st)
-                       : launch_recon_fast_256(p, kB, sBb, sBh, sBr, batch, dtype, st);
+  return rank == 512   ? launch_recon_spec_512(p, kB, sBb, sBh, sBr, batch, dtype, st)
+         : rank == 384 ? launch_recon_spec_384(p, kB, sBb, sBh, sBr, batch, dtype, st)
+                       : launch_recon_spec_256(p, kB, sBb, sBh, sBr, batch, dtype, st);
 }
 
 // The 8-wave kernels (recon_duo_impl.h) for key ranks 256 / 384 / 512 with a separate value basis of rank rv (mode 2; the

@@ -21,18 +21,6 @@
 #include "recon_fast_impl.h"
 #include <utility>
 
-#ifndef XKV_PF
-#define XKV_PF 0
-#endif
-#ifndef XKV_NLR
-#define XKV_NLR 2   // rows of a wave pair's eight that the reconstruction wave loads (the consumer loads the rest)
-#endif
-#ifndef XKV_ORDER
-#define XKV_ORDER 1
-#endif
-#ifndef XKV_ABL
-#define XKV_ABL 0   // timing builds only: bit 0 no softmax / P.A, 1 no transposed reads, 2 no rotation / q-dot, 3 no tile loads, 4 no hand-over
-#endif
 
 namespace xkv {
 namespace spec {
@@ -47,17 +35,12 @@ template <int RK> struct SpecShape {
   static constexpr int NMB = RK / 64;          // 16-feature blocks of the RK / 4 latent features a consumer owns in P.A
   static constexpr int KB_BYTES = 16 * 1024;   // one key buffer: [kq 2][dq 2][part 2][blk 2][lane 64] x 16 bytes of fp16
   static constexpr int SP_FLOATS = 4 * 8 * FSP_ROW;   // one buffer of partial scores: [consumer 4][head 8][FSP_ROW]
-#ifndef XKV_LATE
-#define XKV_LATE (NKS / 4)
-#endif
-#ifndef XKV_EARLY
-#define XKV_EARLY 2
-#endif
-  static constexpr int LATE = XKV_LATE;        // k-steps of a tile that run after the barrier that ends its period
-  static constexpr int EARLY = XKV_EARLY;      // operand reads are issued this many slots before the uniform one-per-slot rate
+  static constexpr int LATE = NKS / 4;         // k-steps of a tile that run after the barrier that ends its period
+  static constexpr int EARLY = 2;              // operand reads are issued this many slots before the uniform one-per-slot rate
+  static constexpr int NLR = 2;                // rows of a wave pair's eight that the reconstruction wave loads (measured: 0, 2, 4, 6, 8)
   // slot of a reconstruction period in which hand-over unit un (0..3) of the previous tile is converted and written
   static constexpr int unit_step(int un) { return LATE + 2 + un * (NKS - LATE - 3) / 4; }
-  static constexpr size_t SHM = (size_t)SRING * FTILE + 2 * KB_BYTES + 2 * SP_FLOATS * 4 + 2 * 8 * 128 * 2 + 128 * 2 + 256;
+  static constexpr size_t SHM = (size_t)SRING * FTILE + 2 * KB_BYTES + 2 * SP_FLOATS * 4 + 2 * 8 * 128 * 2 + 128 * 2;
 };
 
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
@@ -142,12 +125,11 @@ __global__ __launch_bounds__(512) void recon_spec_kernel(const FastParams p) {
   sc_t* qzero = qhat + 2 * 8 * 128;                                        // [128] zeros: the q-dot operand of masked lanes
   const unsigned ring_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)ring;
   if (tid < 128) qzero[tid] = from_f32<sc_t>(0.f);
-  const unsigned pf_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)(qzero + 128);   // 256 bytes nothing reads
 
   // ---- async tile loads: rows 8 wq .. 8 wq + 7 of a tile belong to reconstruction wave wq (the first NLR of them, one behind
   // each of its first MFMA slots) and consumer wq (the rest); one row (RK * 2 bytes: lanes 0 .. RK/8 - 1) per instruction ----
   const int wq = wave & 3;
-  constexpr int NLR = XKV_NLR;
+  constexpr int NLR = S::NLR;
   const unsigned char* Ab = reinterpret_cast<const unsigned char*>(p.kA) + b * p.sAb * 2;
   const int64_t row_bytes = p.sAl * 2;
   const unsigned lane_off = lane * 16;
@@ -174,24 +156,11 @@ __global__ __launch_bounds__(512) void recon_spec_kernel(const FastParams p) {
     constexpr int R0 = decltype(r0_c)::value, R1 = decltype(r1_c)::value;
     static_for<R1 - R0>([&](auto i_c) { issue_one(t, slot_c, IC<R0 + decltype(i_c)::value>(), full_c); });
   };
-#ifdef XKV_STAMP   // timing build: shader-clock stamps of workgroup 0, periods 96..99, behind the lse array
-  long long* stamps = reinterpret_cast<long long*>(p.lse + (int64_t)(p.total_wg / p.hkv) * p.hq);
-  auto now = [&]() -> long long { return __builtin_amdgcn_s_memtime(); };
-  auto put = [&](int pp, int role, int j, long long v) {
-    if (wg == 0 && pp >= 96 && pp < 100 && lane == 0 && (wave == 0 || wave == 4)) stamps[(role * 4 + (pp - 96)) * 8 + j] = v;
-  };
-#else
-  auto now = [&]() -> long long { return 0; };
-  auto put = [&](int, int, int, long long) {};
-#endif
   if (wave < 4) {
     // =================================================================================================================
     // reconstruction wave (kq, dq)
     // =================================================================================================================
     const int kq = wave >> 1, dq = wave & 1;
-#ifdef XKV_PRIO
-    __builtin_amdgcn_s_setprio(XKV_PRIO);
-#endif
     // B operands go from memory straight into accumulation registers (no transit through the 128 ordinary registers the
     // kernel may use): the loads are asm, and so is the wait for them.
     vec8 breg[NKS][2];
@@ -249,20 +218,7 @@ __global__ __launch_bounds__(512) void recon_spec_kernel(const FastParams p) {
       };
       // Past the last tile (and in period 0, which finishes and hands over a tile that does not exist) the same code runs on
       // whatever the LDS holds: nothing downstream uses those results, and one code path keeps the loop a single block.
-      const long long ts0 = now();
-#if XKV_PF > 0
-      // L2 prefetch: the eight workgroups that stream the same rows (one per kv head, one XCD) each touch an eighth of the
-      // cache lines of a tile XKV_PF periods before its loads are issued, so those loads find their lines in the L2
-      if (wave == 0 && lane < 32) {
-        int tok = start + (pp + 2 + XKV_PF) * FT + 4 * (kh & 7) + (lane >> 3);
-        tok = tok < last ? tok : last;
-        // (a load with a register destination would leave that register in flight after the compiler considers it free;
-        // the direct-to-LDS form has no register destination: 4 bytes per lane into 128 spare bytes of the LDS)
-        const unsigned char* line = Ab + (int64_t)tok * row_bytes + (lane & 7) * 128;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(pf_lds), "v"(line) : "memory", "m0");
-      }
-#endif
-      if (pp <= ntiles && !(XKV_ABL & 128)) {   // (timing build bit 7: no reconstruction at all)
+      if (pp <= ntiles) {
         vec8 at[NKS];
         static_for<NKS>([&](auto v_c) {   // slot v of the period: one k-step = two MFMAs
           constexpr int v = decltype(v_c)::value;
@@ -283,25 +239,22 @@ __global__ __launch_bounds__(512) void recon_spec_kernel(const FastParams p) {
           }
           // this wave's share of the loads of tile pp+2, spread evenly over the period: the CU's address unit takes 16 clocks
           // per 1 KiB load, and a wave that issues into a full queue stalls
-          if (!(XKV_ABL & 8) && NLR > 0 && v % (NKS / (NLR > 0 ? NLR : 1)) == (NKS / (NLR > 0 ? NLR : 1)) / 2 && v / (NKS / (NLR > 0 ? NLR : 1)) < NLR) {
+          constexpr int LSTEP = NKS / (NLR > 0 ? NLR : 1);
+          if constexpr (NLR > 0 && v % LSTEP == LSTEP / 2 && v / LSTEP < NLR) {
             XKV_FENCE();
-            issue_one(pp + 2, IC<(u + 2) % 3>(), IC<v / (NKS / (NLR > 0 ? NLR : 1))>(), IC<0>());   // (row clamped to the split: one code path)
+            issue_one(pp + 2, IC<(u + 2) % 3>(), IC<v / LSTEP>(), IC<0>());   // (row clamped to the split: one code path)
             XKV_FENCE();
           }
-          if (!(XKV_ABL & 16)) {
-            if (S::unit_step(0) == v) write_unit(IC<0>());
-            if (S::unit_step(1) == v) write_unit(IC<1>());
-            if (S::unit_step(2) == v) write_unit(IC<2>());
-            if (S::unit_step(3) == v) write_unit(IC<3>());
-          }
+          if (S::unit_step(0) == v) write_unit(IC<0>());
+          if (S::unit_step(1) == v) write_unit(IC<1>());
+          if (S::unit_step(2) == v) write_unit(IC<2>());
+          if (S::unit_step(3) == v) write_unit(IC<3>());
           XKV_FENCE();
         });
 #pragma unroll
         for (int v = 0; v < LATE; ++v) carry[v] = at[NKS - LATE + v];
-        if (NLR > 0 && !(XKV_ABL & 8)) wait_vmcnt<NLR>();   // this wave's rows of tile pp+1 have landed
+        if (NLR > 0) wait_vmcnt<NLR>();   // this wave's rows of tile pp+1 have landed
       }
-      const long long ts1 = now();
-      put(pp, 0, 0, ts0); put(pp, 0, 1, ts1);
       __syncthreads();
     };
     for (int pb = 0; pb < NP6; pb += 6) {
@@ -382,7 +335,8 @@ __global__ __launch_bounds__(512) void recon_spec_kernel(const FastParams p) {
   const int sm_head = n16 & (GP - 1);
   const int sm_row = sm_head < G ? sm_head : G - 1;
   const int sm_tok = 8 * g4 + TPL * (n16 / GP);
-  float m_ref = NEG_INF, l_run = 0.f;   // reference maximum of the lane's head; this lane's share of the head's row sum
+  float m_ref = NEG_INF, l_run = 0.f;   // reference maximum of the lane's head (base-2 domain); this lane's share of its row sum
+  const float scale2 = p.sm_scale * 1.44269504088896f, lazy2 = lazy_rescale<T>() * 1.44269504088896f;
   // P.A accumulators (consumer c owns latent features RK/4 c .. + RK/4; column n16 = head slot) and the transposed tile reads
   // of three tiles live in accumulation registers a[0 .. RK/4), by number (see pa_mfma_at)
   constexpr int TR0 = 4 * NMB, TRSET = 4 * NMB;
@@ -414,10 +368,11 @@ __global__ __launch_bounds__(512) void recon_spec_kernel(const FastParams p) {
     in.q[0] = ld16<sc_vec8>(qrow); in.q[1] = ld16<sc_vec8>(qrow + 32);
     return in;
   };
-  auto stage1_compute = [&](const S1In& in, auto tpar_c) {
+  struct S1Rot { sc_vec8 kop[2]; };
+  auto stage1_rotate = [&](const S1In& in, auto tpar_c) {   // adds the rank halves and rotates: the q-dot's A operands
     constexpr int TPAR = decltype(tpar_c)::value;
     const f16x8 lo = in.k[0] + in.k[1], hi = in.k[2] + in.k[3];
-    f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+    S1Rot r;
 #pragma unroll
     for (int oo = 0; oo < 2; ++oo) {
       h2 lo2[2], hi2[2];
@@ -427,12 +382,17 @@ __global__ __launch_bounds__(512) void recon_spec_kernel(const FastParams p) {
         lo2[e2] = a * ch[TPAR][2 * oo + e2] - bb * sh[TPAR][2 * oo + e2];
         hi2[e2] = bb * ch[TPAR][2 * oo + e2] + a * sh[TPAR][2 * oo + e2];
       }
-      const sc_vec8 kop = {lo2[0][0], lo2[0][1], lo2[1][0], lo2[1][1], hi2[0][0], hi2[0][1], hi2[1][0], hi2[1][1]};
-      // as the A operand of v_mfma_f32_16x16x32, lane (n32, g2) is row n32 % 16 and k-group (n32 / 16) + 2 g2; the B operand
-      // keeps the token halves apart (column c' holds q^ of head c' % 8 in the k-groups of token half c' / 8, zeros elsewhere).
-      // Result: lane (c', g4), register r = score of token 16 (c' / 8) + 4 g4 + r for head c' % 8.
-      sacc = Elem<sc_t>::mfma16(kop, in.q[oo], sacc);
+      r.kop[oo] = sc_vec8{lo2[0][0], lo2[0][1], lo2[1][0], lo2[1][1], hi2[0][0], hi2[0][1], hi2[1][0], hi2[1][1]};
     }
+    return r;
+  };
+  auto stage1_dot = [&](const S1Rot& r, const S1In& in, auto tpar_c) {
+    constexpr int TPAR = decltype(tpar_c)::value;
+    // as the A operand of v_mfma_f32_16x16x32, lane (n32, g2) is row n32 % 16 and k-group (n32 / 16) + 2 g2; the B operand
+    // keeps the token halves apart (column c' holds q^ of head c' % 8 in the k-groups of token half c' / 8, zeros elsewhere).
+    // Result: lane (c', g4), register r = score of token 16 (c' / 8) + 4 g4 + r for head c' % 8.
+    f32x4 sacc = Elem<sc_t>::mfma16(r.kop[0], in.q[0], f32x4{0.f, 0.f, 0.f, 0.f});
+    sacc = Elem<sc_t>::mfma16(r.kop[1], in.q[1], sacc);
     if ((n16 & 7) < G)
       *reinterpret_cast<f32x4*>(s_part + TPAR * SP_FLOATS + (c * 8 + (n16 & 7)) * FSP_ROW + 16 * (n16 >> 3) + 4 * g4) = sacc;
   };
@@ -450,8 +410,12 @@ __global__ __launch_bounds__(512) void recon_spec_kernel(const FastParams p) {
     }
     return in;
   };
-  auto stage23 = [&](int t, const S23In& in, auto ts_c, auto tpar_c) {
+  // (FULL: the tile lies wholly inside the split, no token is masked.)  The softmax runs in the base-2 domain: scores are
+  // scaled by sm_scale * log2(e) in one multiplication and the reference maximum is kept in that domain, so that P is one
+  // subtraction and one v_exp_f32 per score.
+  auto stage23 = [&](int t, const S23In& in, auto ts_c, auto tpar_c, auto full_c) {
     constexpr int TS = decltype(ts_c)::value, TPAR = decltype(tpar_c)::value;
+    constexpr bool FULL = decltype(full_c)::value != 0;
     if (SCORES) {   // consumer c writes heads c and c + 4: lane -> (head c + 4 (lane / 32), token lane % 32)
       const int head = c + 4 * g2;
       const float* sp = s_part + TPAR * SP_FLOATS + (head < G ? head : G - 1) * FSP_ROW + n32;
@@ -474,17 +438,17 @@ __global__ __launch_bounds__(512) void recon_spec_kernel(const FastParams p) {
     float mxl = NEG_INF;
 #pragma unroll
     for (int e = 0; e < TPL; ++e) {
-      s[e] = tok + e < end ? s[e] * p.sm_scale : NEG_INF;
+      s[e] = (FULL || tok + e < end) ? s[e] * scale2 : NEG_INF;
       mxl = fmaxf(mxl, s[e]);
     }
-    // the reference maximum only moves when the tile maximum exceeds it by lazy_rescale<T>(); the cross-lane reduction that
+    // the reference maximum only moves when the tile maximum exceeds it by the lazy bound; the cross-lane reduction that
     // finds the maximum runs only then.  Every consumer sees the same scores, so all four keep the same reference.
-    if (__builtin_amdgcn_ballot_w64(mxl > m_ref + lazy_rescale<T>())) {   // rare: some head's maximum moves
+    if (__builtin_amdgcn_ballot_w64(mxl > m_ref + lazy2)) {   // rare: some head's maximum moves
       float mx = mxl;
 #pragma unroll
       for (int m = GP; m < 64; m <<= 1) mx = fmaxf(mx, __shfl_xor(mx, m));
-      const float m_new = mx > m_ref + lazy_rescale<T>() ? mx : m_ref;
-      const float alpha = __expf(m_ref - m_new);
+      const float m_new = mx > m_ref + lazy2 ? mx : m_ref;
+      const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
       m_ref = m_new;
       l_run *= alpha;
       if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {   // column n16 < GP of the accumulators is this lane's head
@@ -497,7 +461,7 @@ __global__ __launch_bounds__(512) void recon_spec_kernel(const FastParams p) {
     float esum = 0.f;
 #pragma unroll
     for (int k = 0; k < TPL; ++k) {
-      e[k] = __expf(s[k] - m_ref);
+      e[k] = __builtin_amdgcn_exp2f(s[k] - m_ref);
       esum += e[k];
     }
     l_run += esum;
@@ -534,75 +498,42 @@ __global__ __launch_bounds__(512) void recon_spec_kernel(const FastParams p) {
   // STEADY: tiles pp-3 .. pp+2 all exist and tile pp+2 lies wholly inside the split.  Otherwise only the softmax + P.A step is
   // guarded (it must not touch its state for a tile that does not exist); the other steps run on whatever the LDS holds
   // (loads clamp their rows to the split), and nothing uses their results.
+  // The consumer's share of the tile loads is dealt out over the period in four portions: the CU's address unit takes 16
+  // clocks per 1 KiB load, and a wave that issues into a full queue stalls.
   auto period = [&](int pp, auto u_c, auto steady_c) {
     constexpr int u = decltype(u_c)::value;
     constexpr bool STEADY = decltype(steady_c)::value != 0;
+    constexpr int NLC = 8 - NLR, LC1 = NLR + (NLC + 3) / 4, LC2 = NLR + (2 * NLC + 3) / 4, LC3 = NLR + (3 * NLC + 3) / 4;
     const int t_pv = pp - 3;
-    const long long tc0 = now();
-    long long tc1 = 0, tc2 = 0, tc3 = 0, tc4 = 0, tc5 = 0, tc6 = 0, tc7 = 0;
-#ifdef XKV_DUMMY   // interference probe: the consumer does XKV_DUMMY_N units of one kind of work and nothing else
-    {
-      float x = (float)lane;
-#if XKV_DUMMY == 1   // dependent VALU
-      for (int i = 0; i < XKV_DUMMY_N; ++i) asm volatile("v_add_f32 %0, %0, %0" : "+v"(x));
-#elif XKV_DUMMY == 2   // independent VALU (4 chains)
-      float y = x, z = x, w = x;
-      for (int i = 0; i < XKV_DUMMY_N / 4; ++i) asm volatile("v_add_f32 %0, %0, %0\n\tv_add_f32 %1, %1, %1\n\tv_add_f32 %2, %2, %2\n\tv_add_f32 %3, %3, %3" : "+v"(x), "+v"(y), "+v"(z), "+v"(w));
-#elif XKV_DUMMY == 3   // LDS reads of 16 bytes per lane (conflict-free), 8 in flight
-      u32x4 d;
-      for (int i = 0; i < XKV_DUMMY_N / 8; ++i) {
-#pragma unroll
-        for (int k = 0; k < 8; ++k) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(d) : "v"(ring_lds + lane * 16), "n"(k * 1024) : "memory");
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      }
-#elif XKV_DUMMY == 4   // SALU
-      int sx = pp;
-      for (int i = 0; i < XKV_DUMMY_N; ++i) asm volatile("s_add_u32 %0, %0, 1" : "+s"(sx));
-#elif XKV_DUMMY == 5   // independent MFMAs on the consumer's own accumulation registers
-      for (int i = 0; i < XKV_DUMMY_N; ++i) asm volatile("v_mfma_f32_16x16x32_bf16 a[0:3], a[32:35], a[36:39], a[0:3]");
-#endif
-    }
-    __syncthreads();
-    return;
-#endif
+    const bool pv_live = STEADY || (t_pv >= 0 && t_pv < ntiles);
     if (STEADY || pp < ntiles + 3) {
-      // all LDS reads of the period first; the tile loads are issued while they travel
+      // all LDS reads of the period first; the first tile loads are issued while they travel
       const S1In in1 = stage1_load(pp - 2, IC<u & 1>());
       const S23In in23 = stage23_load(IC<(u + 1) & 1>());
       XKV_FENCE();
-      // the consumer's share of the tile loads is dealt out over the period in four portions (see the reconstruction wave)
-      constexpr int NLC = 8 - NLR, LC1 = NLR + (NLC + 3) / 4, LC2 = NLR + (2 * NLC + 3) / 4, LC3 = NLR + (3 * NLC + 3) / 4;
-      if (!(XKV_ABL & 8)) issue_rows(pp + 2, IC<(u + 2) % 3>(), steady_c, IC<NLR>(), IC<LC1>());
-      XKV_FENCE(); tc1 = now(); XKV_FENCE();
-#if XKV_ORDER == 2
-      if (!(XKV_ABL & 4)) stage1_compute(in1, IC<u & 1>());
-#endif
-      if (!SCORES && !(XKV_ABL & 1) && (STEADY || (t_pv >= 0 && t_pv < ntiles))) stage23(t_pv, in23, IC<u % 3>(), IC<(u + 1) & 1>());
-      if (!(XKV_ABL & 8)) issue_rows(pp + 2, IC<(u + 2) % 3>(), steady_c, IC<LC1>(), IC<LC2>());
-      XKV_FENCE(); tc2 = now(); XKV_FENCE();
-      // The compiler does not know of the transposed reads: a wait it placed after them for the key data would wait for them
-      // too.  Using the key data here makes it wait now, and the rotation below then overlaps the transposed reads.
-      asm volatile("" ::"v"(in1.k[0]), "v"(in1.k[1]), "v"(in1.k[2]), "v"(in1.k[3]), "v"(in1.q[0]), "v"(in1.q[1]));
-      if (!(XKV_ABL & 2) && !SCORES) trread(IC<u % 3>(), IC<u % 3>());
-      if (!(XKV_ABL & 8)) issue_rows(pp + 2, IC<(u + 2) % 3>(), steady_c, IC<LC2>(), IC<LC3>());
-      XKV_FENCE(); tc3 = now(); XKV_FENCE();
-#if XKV_ORDER != 2
-      if (!(XKV_ABL & 4)) stage1_compute(in1, IC<u & 1>());
-#endif
-      if (!(XKV_ABL & 8)) issue_rows(pp + 2, IC<(u + 2) % 3>(), steady_c, IC<LC3>(), IC<8>());
-      XKV_FENCE(); tc4 = now(); XKV_FENCE();
+      issue_rows(pp + 2, IC<(u + 2) % 3>(), steady_c, IC<NLR>(), IC<LC1>());
+      XKV_FENCE();
+      // the rotation's VALU work next to the softmax's (independent chains); the q-dot follows the transposed reads
+      const S1Rot rot1 = stage1_rotate(in1, IC<u & 1>());
+      if (!SCORES && pv_live) stage23(t_pv, in23, IC<u % 3>(), IC<(u + 1) & 1>(), steady_c);
+      issue_rows(pp + 2, IC<(u + 2) % 3>(), steady_c, IC<LC1>(), IC<LC2>());
+      XKV_FENCE();
+      // The compiler does not know of the transposed reads: a wait it placed after them for LDS data it read earlier would
+      // wait for them too.  Using that data here makes it wait now, and the q-dot below overlaps the transposed reads.
+      asm volatile("" ::"v"(in1.q[0]), "v"(in1.q[1]), "v"(rot1.kop[0]), "v"(rot1.kop[1]));
+      if (!SCORES) trread(IC<u % 3>(), IC<u % 3>());
+      issue_rows(pp + 2, IC<(u + 2) % 3>(), steady_c, IC<LC2>(), IC<LC3>());
+      XKV_FENCE();
+      stage1_dot(rot1, in1, IC<u & 1>());
+      issue_rows(pp + 2, IC<(u + 2) % 3>(), steady_c, IC<LC3>(), IC<8>());
+      XKV_FENCE();
       if ((u & 1) == 0 && pp >= 2) write_qhat(pp);
-      XKV_FENCE(); tc5 = now(); XKV_FENCE();
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the transposed reads (the compiler does not track them)
-      tc6 = now();
-      if (XKV_ABL & 8) wait_vmcnt<0>(); else if (!(XKV_ABL & 32))
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the transposed reads
       wait_vmcnt<8 - NLR>();      // this wave's rows of tile pp+1 have landed; its loads of tile pp+2 may be in flight
       // Scores mode stores to memory, and stores count in vmcnt like loads: they are issued after the wait, so that they have
       // a whole period to complete before the next one (which cannot tell them from the loads it waits for)
-      if (SCORES && (STEADY || (t_pv >= 0 && t_pv < ntiles))) stage23(t_pv, in23, IC<u % 3>(), IC<(u + 1) & 1>());
-      tc7 = now();
+      if (SCORES && pv_live) stage23(t_pv, in23, IC<u % 3>(), IC<(u + 1) & 1>(), steady_c);
     }
-    put(pp, 1, 0, tc0); put(pp, 1, 1, tc1); put(pp, 1, 2, tc2); put(pp, 1, 3, tc3); put(pp, 1, 4, tc4); put(pp, 1, 5, tc5); put(pp, 1, 6, tc6); put(pp, 1, 7, tc7);
     __syncthreads();
   };
   for (int pb = 0; pb < NP6; pb += 6) {
@@ -631,7 +562,7 @@ __global__ __launch_bounds__(512) void recon_spec_kernel(const FastParams p) {
     float* dst = p.partial + ph * RK + c * (RK / 4) + 4 * g4;
 #pragma unroll
     for (int mb = 0; mb < NMB; ++mb) *reinterpret_cast<f32x4*>(dst + mb * 16) = acc[mb] * inv;
-    if (c == 0 && g4 == 0) p.lse[ph] = m_ref + __logf(l_head);
+    if (c == 0 && g4 == 0) p.lse[ph] = m_ref * 0.6931471805599453f + __logf(l_head);
   }
 }
 
@@ -650,15 +581,6 @@ int launch_recon_spec_t(const FastParams& p, const void* kB, int64_t sBb, int64_
   kern<<<dim3(xcd_grid(total, p.hkv)), dim3(512), S::SHM, st>>>(p);
   return launch_status();
 }
-
-#ifdef XKV_SPEC_DEV_ONE
-template <typename T, int RK>
-int launch_recon_spec_one(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, hipStream_t st) {
-  auto kern = recon_spec_kernel<T, false, RK, 4>;
-  kern<<<dim3(8), dim3(512), SpecShape<RK>::SHM, st>>>(p);
-  return 0;
-}
-#endif
 
 template <int RK>
 int launch_recon_spec_rank(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, int64_t sBr, int batch, int dtype,

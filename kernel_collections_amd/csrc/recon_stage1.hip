@@ -19,7 +19,6 @@
 #include "xkv_common.h"
 #include "recon_fast.h"
 #include <mutex>
-#include <cstdlib>
 
 namespace xkv {
 
@@ -414,12 +413,10 @@ extern "C" int xkv_recon_stage1(const void* q_pe, xkv_kv_operand kA, const void*
     f.num_splits = num_kv_splits; f.kv_lens = kv_lens;
     f.hq = hq; f.hkv = hkv; f.kv_len = kv_len; f.max_splits = max_splits; f.total_wg = batch * hkv * max_splits;
     f.sm_scale = sm_scale; f.inv_freq = inv_freq; f.pos_offset = pos_offset;
-    static const char* form = getenv("XKV_RECON_FORM");
-    if (!(form && form[0] == 'f'))
-      return rank == 512   ? launch_recon_spec_512(f, kB, sBb, sBh, sBr, batch, dtype, st)
-             : rank == 384 ? launch_recon_spec_384(f, kB, sBb, sBh, sBr, batch, dtype, st)
-                           : launch_recon_spec_256(f, kB, sBb, sBh, sBr, batch, dtype, st);
-    return launch_recon_fast(f, kB, sBb, sBh, sBr, batch, dtype, rank, st);
+    // Scores only at rank 256: the 4-wave kernel, the one instantiation small enough for two workgroups per CU (measured
+    // 10 - 15 % ahead there).  Everything else: the wave-specialised kernel (8 - 13 % ahead of the 4-wave kernel).
+    if (!(so && rank == 256)) return launch_recon_spec(f, kB, sBb, sBh, sBr, batch, dtype, rank, st);
+    return launch_recon_fast_256(f, kB, sBb, sBh, sBr, batch, dtype, st);
   }
   // 8-wave kernels: a value basis of its own beside key ranks 256 / 384 / 512
   if (!so && !vshared && rope && !sin_cos && hq / hkv <= 8 && workspace && need > 0 && workspace_bytes >= need &&
