@@ -48,7 +48,8 @@ enum {
   XKV_EUNSUPPORTED = -2,/* shape outside the built envelope (see each function) */
   XKV_EALIGN = -3,      /* stride or pointer not 16-byte aligned */
   XKV_EDTYPE = -4,
-  XKV_ESCRATCH = -5     /* xkv_recon_stage1_static: needs more than XKV_STATIC_SCRATCH_BYTES */
+  XKV_ESCRATCH = -5,    /* xkv_recon_stage1_static: needs more than XKV_STATIC_SCRATCH_BYTES */
+  XKV_ETOOLCHAIN = -6   /* this build of a kernel that tracks its own loads spills registers: rebuild with the validated compiler */
 };
 
 int xkv_abi_version(void);
@@ -202,6 +203,10 @@ int64_t xkv_recon_workspace_bytes(int batch, int hkv, int rank, int64_t stride_k
  * stride_kB_b == 0) returns XKV_ESCRATCH and launches nothing.  Every call on a GPU uses that GPU's one array and
  * overwrites what the previous call left there: calls on the same GPU must not overlap (two streams, two threads) - they
  * would race on it; calls in stream order on one stream are safe.  The device current at the call must be the stream's.
+ * The FIRST call on a device for a given kernel shape does host-side set-up (the array's address is looked up with
+ * hipGetSymbolAddress, the kernel's dynamic LDS size is raised with hipFuncSetAttribute): make one warm-up call per device
+ * and shape outside stream capture before capturing.  XKV_ESCRATCH is returned only for shapes that would take a path that
+ * packs kB (generated RoPE angles, at most 8 query heads per kv head); other shapes run the generic kernel without scratch.
  * No counterpart in the reference, whose wrappers allocate with torch.empty on every call
  * (flash_recontruction/fused_attention/no_pe/v1.py:434-446). */
 #define XKV_STATIC_SCRATCH_BYTES (4 << 20)

@@ -21,6 +21,7 @@ EXPORTS = (
 )
 STATIC_SCRATCH_BYTES = 4 << 20
 XKV_ESCRATCH = -5
+XKV_ETOOLCHAIN = -6
 
 
 class KVOperand(Structure):

@@ -18,7 +18,7 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-inline-asm",
 ]
-# Per-file additions.  the recon_fast_*.hip and recon_duo_*.hip units: MFMA results must land in ordinary VGPRs (the RoPE / softmax VALU code reads
+# Per-file additions.  the recon_fast_*.hip, recon_spec_*.hip and recon_duo_*.hip units: MFMA results must land in ordinary VGPRs (the RoPE / softmax VALU code reads
 # them; with accumulation-register results every value costs a v_accvgpr_read), while the stationary B operands are
 # pinned to accumulation registers by the source itself.
 _VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
@@ -26,6 +26,27 @@ EXTRA_FLAGS = {
     "recon_fast_256.hip": _VGPR_FORM,
     "recon_duo_b.hip": _VGPR_FORM, "recon_duo_c.hip": _VGPR_FORM, "recon_spec_512.hip": _VGPR_FORM, "recon_spec_384.hip": _VGPR_FORM, "recon_spec_256.hip": _VGPR_FORM,
 }
+
+
+# The compiler the kernels were validated with.  latent_ring.hip, recon_fast / recon_duo / recon_spec issue loads in asm
+# and track their completion by hand; that is correct for the register allocation this compiler produces and is re-checked
+# by tests/test_gpu_ring_forms.py and the parity suite.  Another compiler builds, with a loud warning: run those tests on a
+# GPU before trusting it.  (At run time the library refuses such a kernel outright if its build spills registers.)
+VALIDATED_HIPCC = "roc-7.2.0 26014"
+
+
+def _check_compiler() -> None:
+    try:
+        out = subprocess.run([HIPCC, "--version"], capture_output=True, text=True).stdout
+    except OSError as e:   # pragma: no cover
+        raise RuntimeError(f"cannot run {HIPCC}: {e}")
+    if VALIDATED_HIPCC not in out:
+        line = next((l for l in out.splitlines() if "clang version" in l), out.strip()[:120])
+        sys.stderr.write(
+            "\n*** kernel_collections_amd.build: hipcc is not the validated one (%s); found: %s\n"
+            "*** the kernels that track their own loads (latent_ring, recon_fast, recon_duo, recon_spec) must be re-checked:\n"
+            "***   python -m pytest tests/test_gpu_ring_forms.py tests/test_gpu_parity.py tests/test_gpu_peaked.py -m gpu\n\n"
+            % (VALIDATED_HIPCC, line))
 
 
 def sources():
@@ -46,6 +67,7 @@ def _compile(src: str) -> str:
 
 def build(verbose: bool = True) -> str:
     """Compile every kernel source and link the shared library; always recompiles."""
+    _check_compiler()
     os.makedirs(OBJ, exist_ok=True)
     srcs = sources()
     with cf.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:

@@ -125,8 +125,8 @@ static int launch_stream(const void* src, int64_t bytes, int wgs, float* out, hi
   auto kern = ceiling_stream_kernel<TO_LDS, DEPTH>;
   if (TO_LDS) {
     static DynLds lds;
-    hipError_t e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), (int)shm);
-    if (e != hipSuccess) return (int)e;
+    const int e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), (int)shm);
+    if (e != XKV_OK) return e;
   }
   kern<<<dim3(wgs), dim3(256), shm, st>>>(reinterpret_cast<const unsigned char*>(src), steps, out);
   return launch_status();

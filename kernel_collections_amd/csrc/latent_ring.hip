@@ -557,8 +557,8 @@ static int launch_ring_t(const RingParams& p, int batch, hipStream_t st) {
   constexpr int SHM = RingShape<TN, DN, HAS_R, VMODE, NHB, DVW>::shm(LO);
   auto kern = latent_ring_kernel<T, TN, NHB, LO, DN, HAS_R, VMODE, DVW>;
   static DynLds lds;
-  hipError_t e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), SHM);
-  if (e != hipSuccess) return (int)e;
+  const int e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), SHM, true);
+  if (e != XKV_OK) return e;
   const int total = batch * p.groups * p.max_splits;
   kern<<<dim3(xcd_grid(total, p.groups)), dim3(512), SHM, st>>>(p);
   return launch_status();

@@ -336,8 +336,8 @@ static int launch_latent(const LatentParams& p, int batch, hipStream_t st) {
   if (shm > 160 * 1024) return XKV_EUNSUPPORTED;
   auto kern = latent_stage1_kernel<T, NHB, TN, NVB_MAX, NPK_C, NPK_R, NPK_V, VSHARED, SCORES_ONLY>;
   static DynLds lds;
-  hipError_t e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), (int)shm);
-  if (e != hipSuccess) return (int)e;
+  const int e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), (int)shm);
+  if (e != XKV_OK) return e;
   const int total = batch * p.groups * p.max_splits;
   const int grid = xcd_grid(total, p.groups);
   kern<<<dim3(grid), dim3(256), shm, st>>>(p);

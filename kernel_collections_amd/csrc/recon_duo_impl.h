@@ -482,8 +482,8 @@ int launch_duo_t(const FastParams& p, const void* kB, int64_t sBb, int64_t sBh, 
   duo_pack_b_kernel<T, RK><<<dim3(p.hkv, nb, 16), dim3(256), 0, st>>>((const T*)kB, (T*)p.Bp, sBb, sBh, sBr, p.hkv);
   auto kern = recon_duo_kernel<T, RK, RV, MODE>;
   static DynLds lds;
-  hipError_t e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), S::SHM);
-  if (e != hipSuccess) return (int)e;
+  const int e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), S::SHM, true);
+  if (e != XKV_OK) return e;
   const int total = batch * p.hkv * p.max_splits;
   kern<<<dim3(xcd_grid(total, p.hkv)), dim3(64 * NW), S::SHM, st>>>(p);
   return launch_status();

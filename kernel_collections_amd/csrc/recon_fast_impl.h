@@ -574,8 +574,8 @@ int launch_recon_fast_t(const FastParams& p, const void* kB, int64_t sBb, int64_
   pack_b_kernel<T, RK><<<dim3(p.hkv, nb, 32), dim3(256), 0, st>>>((const T*)kB, (T*)p.Bp, sBb, sBh, sBr, p.hkv);
   auto kern = p.scores ? recon_fast_kernel<T, true, RK> : recon_fast_kernel<T, false, RK>;
   static DynLds lds[2];
-  hipError_t e = ensure_dynamic_lds(lds[p.scores ? 1 : 0], reinterpret_cast<const void*>(kern), (int)S::SHM);
-  if (e != hipSuccess) return (int)e;
+  const int e = ensure_dynamic_lds(lds[p.scores ? 1 : 0], reinterpret_cast<const void*>(kern), (int)S::SHM, true);
+  if (e != XKV_OK) return e;
   const int total = batch * p.hkv * p.max_splits;
   kern<<<dim3(xcd_grid(total, p.hkv)), dim3(256), S::SHM, st>>>(p);
   return launch_status();

@@ -575,8 +575,8 @@ int launch_recon_spec_t(const FastParams& p, const void* kB, int64_t sBb, int64_
   auto kern = p.scores ? (gp4 ? recon_spec_kernel<T, true, RK, 4> : recon_spec_kernel<T, true, RK, 8>)
                        : (gp4 ? recon_spec_kernel<T, false, RK, 4> : recon_spec_kernel<T, false, RK, 8>);
   static DynLds lds[4];
-  hipError_t e = ensure_dynamic_lds(lds[(p.scores ? 2 : 0) + (gp4 ? 1 : 0)], reinterpret_cast<const void*>(kern), (int)S::SHM);
-  if (e != hipSuccess) return (int)e;
+  const int e = ensure_dynamic_lds(lds[(p.scores ? 2 : 0) + (gp4 ? 1 : 0)], reinterpret_cast<const void*>(kern), (int)S::SHM, true);
+  if (e != XKV_OK) return e;
   const int total = batch * p.hkv * p.max_splits;
   kern<<<dim3(xcd_grid(total, p.hkv)), dim3(512), S::SHM, st>>>(p);
   return launch_status();

@@ -330,8 +330,8 @@ static int launch_recon(const ReconParams& p, int batch, hipStream_t st) {
   shm += 4 * 16 * (RTN + 4) * 4 + 16 * (RTN + 8) * 2 + 16 * 4 + 16 * 8;
   auto kern = recon_stage1_kernel<T, NKS, EXACT, NVB_MAX, VSHARED, SCORES_ONLY>;
   static DynLds lds;
-  hipError_t e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), (int)shm);
-  if (e != hipSuccess) return (int)e;
+  const int e = ensure_dynamic_lds(lds, reinterpret_cast<const void*>(kern), (int)shm);
+  if (e != XKV_OK) return e;
   const int total = batch * p.hkv * p.max_splits;
   kern<<<dim3(xcd_grid(total, p.hkv)), dim3(256), shm, st>>>(p);
   return launch_status();
@@ -475,7 +475,10 @@ extern "C" int xkv_recon_stage1_static(const void* q_pe, xkv_kv_operand kA, cons
                                        const float* inv_freq, int64_t pos_offset, const void* sin_cos,
                                        int64_t sc_stride_l, int dtype, void* stream) {
   if (batch <= 0 || hkv <= 0) return XKV_EINVAL;
-  const int64_t need = xkv_recon_workspace_bytes(batch, hkv, kA.dim, sBb);
+  int64_t need = xkv_recon_workspace_bytes(batch, hkv, kA.dim, sBb);
+  // only the MFMA-bound paths (generated angles, at most 8 query heads per kv head) pack kB; every other shape runs the
+  // generic kernel, which needs no scratch
+  if (!(rope && !sin_cos && hq > 0 && hq % hkv == 0 && hq / hkv <= 8)) need = 0;
   if (need > (int64_t)XKV_STATIC_SCRATCH_BYTES) return XKV_ESCRATCH;   // nothing is launched
   void* ws = nullptr;
   if (need > 0) {

@@ -364,8 +364,16 @@ static int launch_merge(const float* partial, const float* lse, void* out, const
   // is an up-projection, whose vB rows then weigh more than the partial rows
   const int g = hq / hkv;
   const bool enough_wgs = vB && (int64_t)hkv * batch >= 128;   // vB costs more than the partial rows: keep it read once per kv head
-  const int hpw = (g > 16 || (max_splits > 16 && !enough_wgs)) ? 1 : g;
+  int hpw = (g > 16 || (max_splits > 16 && !enough_wgs)) ? 1 : g;
+  // dynamic LDS beside the kernel's 8 KiB of static LDS: the default limit of 64 KiB per workgroup must hold both; a group
+  // of heads that does not fit is merged one head per workgroup, and a single head that does not fit is refused
+  constexpr size_t LDS_LIMIT = 64 * 1024, STATIC_LDS = 8 * 1024;
   size_t shm = (size_t)hpw * (dv + max_splits) * sizeof(float);
+  if (shm + STATIC_LDS > LDS_LIMIT) {
+    hpw = 1;
+    shm = (size_t)(dv + max_splits) * sizeof(float);
+    if (shm + STATIC_LDS > LDS_LIMIT) return XKV_EUNSUPPORTED;
+  }
   // a small grid over many splits is bound by the latency of its partial-row loads: split the up-projection's columns
   // over more workgroups
   int zb = 1;
@@ -501,6 +509,7 @@ extern "C" const char* xkv_error_string(int code) {
     case XKV_EALIGN: return "pointer or stride not 16-byte aligned";
     case XKV_EDTYPE: return "unsupported dtype code";
     case XKV_ESCRATCH: return "the call needs more scratch than the library's static device array holds";
+    case XKV_ETOOLCHAIN: return "a kernel that tracks its own loads was built with register spills: rebuild with the validated compiler";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown xkv error";
   }
 }

@@ -138,14 +138,24 @@ struct DynLds {
   std::atomic<int> bytes[16];
   DynLds() { for (auto& b : bytes) b.store(0, std::memory_order_relaxed); }
 };
-inline hipError_t ensure_dynamic_lds(DynLds& st, const void* kernel, int bytes) {
+// `hand_tracked`: the kernel issues loads in asm and tracks their completion by hand (s_waitcnt counts, registers that
+// stay in flight across instructions).  That bookkeeping only holds while the compiler adds no memory traffic of its own to
+// the kernel: a build whose register allocation spills (another compiler, other flags) is refused with XKV_ETOOLCHAIN
+// instead of computing on stale registers.  Returns XKV_OK, XKV_ETOOLCHAIN or a positive hipError_t.
+inline int ensure_dynamic_lds(DynLds& st, const void* kernel, int bytes, bool hand_tracked = false) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  if (dev >= 0 && dev < 16 && st.bytes[dev].load(std::memory_order_acquire) >= bytes) return hipSuccess;
+  if (e != hipSuccess) return (int)e;
+  if (dev >= 0 && dev < 16 && st.bytes[dev].load(std::memory_order_acquire) >= bytes) return XKV_OK;
+  if (hand_tracked) {
+    hipFuncAttributes attr;
+    e = hipFuncGetAttributes(&attr, kernel);
+    if (e != hipSuccess) return (int)e;
+    if (attr.localSizeBytes != 0) return XKV_ETOOLCHAIN;
+  }
   e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
   if (e == hipSuccess && dev >= 0 && dev < 16) st.bytes[dev].store(bytes, std::memory_order_release);
-  return e;
+  return (int)e;
 }
 
 inline int launch_status() {

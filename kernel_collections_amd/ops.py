@@ -155,6 +155,9 @@ def absorb_q(q3: torch.Tensor, Bk: torch.Tensor, want_lo: bool = True) -> Tuple[
     """q3 `[b,Hq,d]`, Bk `[b,Hkv,r,d]` (any batch/head/rank strides) -> q~ hi (and lo) `[b,Hq,r]`."""
     b, hq, d = q3.shape
     _, hkv, r, _ = Bk.shape
+    if hkv == 1 and hq > 32:   # the kernel serves at most 32 query heads per kv head: one shared matrix seen as several heads
+        hkv = head_groups(hq)
+        Bk = Bk.expand(-1, hkv, -1, -1)
     Bk = as_rows(Bk)
     hi = torch.empty((b, hq, r), dtype=q3.dtype, device=q3.device)
     lo = torch.empty_like(hi) if want_lo else None
@@ -236,6 +239,9 @@ def merge_stage2(partial, lse, out, vB, num_kv_splits, kv_lens, batch, hq, hkv, 
     if vB is None:
         call(out, None, dv, (0, 0, 0), _lib.XKV_BF16, lse_out)
         return out
+    if hkv == 1 and hq > 32:   # at most 32 query heads per kv head in the up-projecting merge: the shared matrix as several heads
+        hkv = head_groups(hq)
+        vB = vB.expand(-1, hkv, -1, -1)
     vB = as_rows(vB)
     sv, vdt = (vB.stride(0), vB.stride(1), vB.stride(2)), dtype_code(vB.dtype)
     for c0 in range(0, vB.shape[-1], 512):

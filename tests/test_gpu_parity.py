@@ -108,7 +108,7 @@ def test_qab_nope_shared_factor_stride0_and_row_strides(dev):
 @pytest.mark.parametrize("dtype", [BF, FP])
 @pytest.mark.parametrize("b,hq,hkv,L,r,theta", [(2, 32, 8, 1000, 512, 5e5), (1, 8, 2, 77, 256, 1e7),
                                                 (1, 16, 1, 2085, 384, 1e4), (2, 4, 4, 40, 192, 1e7),
-                                                (2, 8, 2, 300, 384, 5e5),    # 4-wave kernel at rank 384, scores mode
+                                                (2, 8, 2, 300, 384, 5e5),    # wave-specialised kernel at rank 384, scores mode
                                                 (1, 16, 2, 1500, 256, 1e7)])  # ... at rank 256, 8 heads per kv head
 def test_qab_rope(dev, dtype, b, hq, hkv, L, r, theta):
     d = 128
@@ -216,7 +216,7 @@ def test_fused_rope(dev, dtype, b, hq, hkv, L, rk, rv, S, shared):
     (1, 24, 8, 256, 512, False, [1500], 7, 0),             # the last splits are dead
     (2, 32, 8, 384, 384, True, [900, 1200], 4, 0),
     (2, 16, 4, 256, 256, True, [33, 4000], 6, 131072 - 4000),
-    (1, 16, 2, 384, 384, True, [1500], 3, 0),              # the 4-wave kernel at ranks 384 / 256: 8 heads per kv head ...
+    (1, 16, 2, 384, 384, True, [1500], 3, 0),              # the wave-specialised kernel at ranks 384 / 256: 8 heads per kv head ...
     (2, 8, 8, 256, 256, True, [100, 257], 2, 50000)])      # ... and one
 @pytest.mark.parametrize("form", ["fused", "two_pass", "as_shipped"])
 def test_fused_rope_wide_kernels(dev, dtype, b, hq, hkv, rk, rv, shared, lens, S, off, form, monkeypatch):
@@ -364,6 +364,18 @@ def test_mla_many_heads(dev):
         gen((b, L, 1, c), std=1 / 3, seed=3), gen((b, L, 1, e), std=1 / 3, seed=4)
     ref = oracle.mla_ref(*f32(qn, qr, ckv, kpe), 0.1)
     check_out(mla2.mla_decode_attention_fwd(*dev_(dev, qn, qr, ckv, kpe), 0.1), ref)
+
+
+@pytest.mark.parametrize("b,H", [(2, 128), (1, 64), (1, 48)])
+def test_mla2_xkv_many_heads(dev, b, H):
+    """More than 32 heads share the one factor matrix: the absorb and the up-projecting merge see it as head groups of <= 32."""
+    L, c, e, r = 600, 512, 64, 256
+    qn, qr, kpe = gen((b, H, c), std=1 / 3, seed=1), gen((b, H, e), std=1 / 3, seed=2), gen((b, L, 1, e), std=1 / 3, seed=4)
+    kvA, kvB = gen((b, L, 1, r), std=1 / 3, seed=5), gen((b, 1, r, c), std=r ** -0.5, seed=6)
+    ref = oracle.mla_xkv_ref(*f32(qn, qr, kvA, kvB, kpe), 0.1)
+    out = mla2.mla_decode_attention_xKV(*dev_(dev, qn, qr, kvA, kvB, kpe), 0.1)
+    assert out.shape == (b, H, c)
+    check_out(out, ref, "mla2 xKV, %d heads" % H)
 
 
 @pytest.mark.parametrize("dk,dv,hkv", [(384, 384, 1), (576, 512, 1), (288, 256, 2), (128, 128, 4)])

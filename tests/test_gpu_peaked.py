@@ -107,8 +107,8 @@ class ReconRope(Path):
             return 0.0
         ang = torch.outer(torch.arange(self.off, self.off + self.L).double(), oracle.rope_inv_freq(D, self.theta).double())
         ang = torch.cat((ang, ang), -1)
-        exact = self.ref(q, dict(i, cos=ang.cos().float(), sin=ang.sin().float()))
-        return (exact - ref).abs().max().item()
+        self.exact = self.ref(q, dict(i, cos=ang.cos().float(), sin=ang.sin().float()))
+        return (self.exact - ref).abs().max().item()
 
 
 class FusedNope(Path):
@@ -133,8 +133,8 @@ class FusedNope(Path):
 
 
 class Plain(Path):
-    def __init__(self, v_factorised):
-        self.vf = v_factorised
+    def __init__(self, v_factorised, hkv=8):
+        self.vf, self.hkv = v_factorised, hkv
 
     def inputs(self, dtype):
         return dict(K=gen((self.b, self.L, self.hkv, D), dtype=dtype, seed=2), V=gen((self.b, self.L, self.hkv, D), dtype=dtype, seed=3),
@@ -178,11 +178,12 @@ class Mla(Path):
 
 
 PATHS = {
-    "recon_fast(r512 shared)": ReconRope(512, 512, True),
-    "recon_fast(r512 shared, positions near 128K)": ReconRope(512, 512, True, off=131072 - 1500),
+    "recon_spec(r512 shared)": ReconRope(512, 512, True),
+    "recon_spec(r512 shared, positions near 128K)": ReconRope(512, 512, True, off=131072 - 1500),
+    "recon_spec(r384 shared)": ReconRope(384, 384, True),
     "recon_duo(r384/512)": ReconRope(384, 512, False),
     "recon_duo(r512/512)": ReconRope(512, 512, False),
-    "recon_fast(r256 shared, G 8)": ReconRope(256, 256, True, hq=16, hkv=2),
+    "recon_spec(r256 shared, G 8)": ReconRope(256, 256, True, hq=16, hkv=2),
     "recon_stage1(r192 shared)": ReconRope(192, 192, True),
     "recon_stage1(r512 table)": ReconRope(512, 512, True, table=True),
     "latent_ring(absorbed r512/512)": FusedNope(512, 512),
@@ -190,7 +191,8 @@ PATHS = {
     "latent_stage1(absorbed r192/64)": FusedNope(192, 64),
     "latent_ring(mla 512+64)": Mla(),
     "latent_ring(block-diagonal q, v_A 512)": Plain(True),
-    "latent_stage1(plain gqa)": Plain(False),
+    "latent_ring(plain gqa, 8 kv heads as one row)": Plain(False),
+    "latent_stage1(plain gqa, 4 kv heads)": Plain(False, hkv=4),
 }
 
 
@@ -209,5 +211,13 @@ def test_peaked_softmax(dev, name, scn, dtype):
     if noise == 0.0:
         check_out(out, ref, f"{name} / {scn}")
     else:
-        err = max_abs(out, ref)
-        assert err <= OUT_ATOL + 1.5 * noise, f"{name} / {scn}: max abs err {err:.3e} (oracle's own angle noise {noise:.3e})"
+        # Near position 128K an fp32 angle fl(pos * inv_freq) is off the exact one by up to 4e-3 rad.  The oracle rounds it at
+        # every token, the kernel at the base of every 30th tile (and adds small, exact in-tile angles): both are about
+        # `noise` away from the result at exact angles, in different directions.  So the kernel is held to the contract's
+        # 2e-2 plus ONCE the noise against the exact-angle oracle, and plus TWICE the noise against the fp32-angle oracle
+        # (the two deviations add).  All three figures are printed (pytest -s).
+        err, err_exact = max_abs(out, ref), max_abs(out, p.exact)
+        print(f"\n{name} / {scn} / {dtype}: max abs err {err:.3e} vs the fp32-angle oracle, {err_exact:.3e} vs exact angles, "
+              f"oracle's own angle noise {noise:.3e}")
+        assert err_exact <= OUT_ATOL + noise, f"{name} / {scn}: {err_exact:.3e} from the exact-angle result (noise {noise:.3e})"
+        assert err <= OUT_ATOL + 2 * noise, f"{name} / {scn}: max abs err {err:.3e} (oracle's own angle noise {noise:.3e})"
