@@ -28,13 +28,41 @@ sys.path.insert(0, ROOT)
 # published peaks of the MI355X, the denominators of roofline.frac
 PEAK_HBM_GBS = 8000.0
 PEAK_BF16_TFLOPS = 2500.0
-# HBM bytes of one stage-1 launch at the default c3 shape, from two rocprofv3 --pmc runs of this file
-# (FETCH_SIZE, WRITE_SIZE; each scaled by what the counter reads for --calib-copy's 512 MiB copies).
-# A counter cannot be read from inside the timed process, so the figure is recorded here.
-C3_STAGE1_HBM_BYTES = 537274 * 1024     # recon_fast_kernel 2 x 266578.5 + 2056.0 KiB, pack_b_kernel 2 x 518.5 + 1024 KiB
-C5_RING_HBM_BYTES = 604800 * 1024       # same method, latent_ring_kernel at the default c5 shape (2 x 298272.1 + 8256.0 KiB)
-C2_RING_HBM_BYTES = 151785 * 1024       # latent_ring_kernel, scores mode, default c2 shape (2 x 67700.4 + 16384.0 KiB)
-C4_RING_HBM_BYTES = 3022744 * 1024      # latent_ring_kernel at c4 plain with the planned split length (2 x 1509401.8 + 3940.0 KiB)
+# roofline.traffic: HBM bytes of one launch of a workload's dominant kernel, from two rocprofv3 --pmc runs of this file
+# (FETCH_SIZE, WRITE_SIZE; each scaled by what the counter reads for --calib-copy's 512 MiB copies).  A counter cannot be read
+# from inside the timed process, so the figures are kept in profiles/hbm_traffic_table.txt, one line per workload:
+#   <workload> <bytes> <kernel source file>:<first 16 hex digits of its sha256> ...
+# A figure is reported only while every source file it names still has the recorded hash: after a kernel change the line
+# reads null until the counters have been collected again (`bench.py --traffic-line <workload> <bytes>` prints a fresh line).
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_table.txt")
+CSRC = os.path.join(ROOT, "kernel_collections_amd", "csrc")
+TRAFFIC_SOURCES = {
+    "c3": ["recon_spec_impl.h", "recon_fast_impl.h", "recon_stage1.hip"],
+    "c2": ["latent_ring.hip", "latent_ring.h"], "c5": ["latent_ring.hip", "latent_ring.h"], "c4": ["latent_ring.hip", "latent_ring.h"],
+}
+
+
+def _source_hash(name):
+    import hashlib
+    return hashlib.sha256(open(os.path.join(CSRC, name), "rb").read()).hexdigest()[:16]
+
+
+def traffic_line(workload, nbytes):
+    return " ".join([workload, str(int(nbytes))] + ["%s:%s" % (f, _source_hash(f)) for f in TRAFFIC_SOURCES[workload]])
+
+
+def recorded_traffic(workload):
+    try:
+        rows = [l.split() for l in open(TRAFFIC_TABLE) if l.strip() and not l.startswith("#")]
+    except OSError:
+        return None
+    for row in rows:
+        if row[0] == workload:
+            ok = all(_source_hash(f) == h for f, h in (x.split(":") for x in row[2:]))
+            return int(row[1]) if ok else None
+    return None
+
+
 OUT_ATOL, SCORE_RTOL = 2e-2, 1e-2     # the parity bars (attention output max-abs, scores max|delta| / max|ref|)
 
 
@@ -151,7 +179,53 @@ def device_info(dev):
         info["memory_clock_mhz"], info["memory_bus_bits"] = round(mem_mhz), int(bus)
         info["derived_hbm_peak_gbs"] = round(mem_mhz * 1e6 * 2 * bus / 8 / 1e9, 1)   # double data rate
     info["hbm_gib"] = round(p.total_memory / 2 ** 30, 1)
+    if not mhz:
+        info["clock_note"] = "this torch build exposes no clock attribute; see roofline.sustained_mfma_clock_mhz (c3) and sysfs"
+    info["sysfs"] = sysfs_gpu_state()
     return info
+
+
+def sysfs_gpu_state():
+    """Clock and power figures the driver exposes through sysfs, read best-effort (an ordinary user may read them on most
+    installations): the engine clock level in force and the power cap / draw.  None where the files are absent."""
+    import glob
+    out = {}
+    for card in sorted(glob.glob("/sys/class/drm/card[0-9]*/device")):
+        try:
+            lines = open(os.path.join(card, "pp_dpm_sclk")).read().split("\n")
+        except OSError:
+            continue
+        cur = [l for l in lines if l.strip().endswith("*")]
+        out["sclk_levels"] = [l.strip() for l in lines if l.strip()][:4]
+        if cur:
+            out["sclk_in_force"] = cur[0].strip()
+        for name, key in (("power1_cap", "power_cap_w"), ("power1_average", "power_draw_w"), ("power1_input", "power_draw_w")):
+            for f in glob.glob(os.path.join(card, "hwmon", "hwmon*", name)):
+                try:
+                    out[key] = round(int(open(f).read().strip()) / 1e6, 1)
+                except (OSError, ValueError):
+                    pass
+        break
+    return out or None
+
+
+def sustained_mfma(dev, seconds=0.05):
+    """What this box sustains right now with nothing but v_mfma_f32_32x32x16_bf16 on every SIMD (two waves each): the kernel
+    of `--config ceilings`, run for about `seconds` after the same settling as the workload.  Also the clock that rate
+    implies (4096 dense bf16 FLOP per clock and CU), which is the clock the power manager grants under matrix load."""
+    from kernel_collections_amd import _lib, ops
+    lib = _lib.lib()
+    cus = ops.num_cus(dev)
+    st = _lib.stream_ptr(torch.empty(1, device=dev))
+    out = torch.empty(cus * 2 * 256, dtype=torch.float32, device=dev)
+    iters, wgs = 2000, cus * 2
+    fn = lambda i: _lib.check(lib.xkv_ceiling_mfma(_lib.ptr(out), wgs, iters, _lib.XKV_BF16, st), "xkv_ceiling_mfma")
+    flop = wgs * 4 * iters * 32 * 32768
+    _settle(fn)
+    n = max(3, int(seconds / (flop / 1.8e15)))
+    avg_ms, _ = time_kernel(fn, n, 2, settle=False)
+    tf = flop / (avg_ms * 1e-3) / 1e12
+    return round(tf, 1), round(tf * 1e12 / (cus * 4096) / 1e6)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -204,6 +278,8 @@ def bench_c3(args, dev):
     flops = B * L * (2 * r * Hkv * d + 2 * Hq * d + 2 * Hq * r)
     achieved = flops / (k_avg_ms * 1e-3) / 1e12
     algo_bytes = B * L * r * 2 + 2 * r * Hkv * d * 2
+    # the same box's MFMA ceiling, measured next to the kernel: tells a slower box from a slower kernel
+    sus_tf, sus_mhz = sustained_mfma(dev)
 
     # the same workload with a value basis of its own (A_v distinct from A)
     distinct = None
@@ -216,7 +292,7 @@ def bench_c3(args, dev):
         parity["distinct_value_basis"] = require_close(o2[:1], ref_d, "c3 with its own value basis, sequence 0")
         d_ms, d_q = time_loop(lambda i: fr.gqa_xKV_rope(q[i % layers], A, kB[i % layers], Av, vB[i % layers], o2, ns, S, scale, theta),
                               args.steps, args.warmup)
-        distinct = {"us": round(d_ms * 1e3 / args.steps, 2), "step_us": d_q, "kernel": "recon_fast_kernel (scores) + latent_ring_kernel (given scores), two passes",
+        distinct = {"us": round(d_ms * 1e3 / args.steps, 2), "step_us": d_q, "kernel": "recon_spec_kernel (scores) + latent_ring_kernel (given scores), two passes",
                     "hbm_bytes": 2 * B * L * r * 2}
         del Av
 
@@ -245,11 +321,13 @@ def bench_c3(args, dev):
         "tokens_per_s": B / (us * 1e-6), "kv_tokens_scanned_per_s": B * L / (us * 1e-6),
         "config": {"workload": "c3 fused RoPE xKV decode: batch 16, 32q/8kv heads, d128, ctx %d, rank 512, "
                                "A shared by K/V and by a 4-layer group, per layer" % L, "kv_splits": S},
-        "roofline": {"bound": "mfma", "kernel": "recon_fast_kernel", "achieved": round(achieved, 1),
+        "roofline": {"bound": "mfma", "kernel": "recon_spec_kernel", "achieved": round(achieved, 1),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-                     "traffic": C3_STAGE1_HBM_BYTES if (L == 32768 and not args.splits) else None,
+                     "traffic": recorded_traffic("c3") if (L == 32768 and not args.splits) else None,
                      "kernel_avg_us": round(k_avg_ms * 1e3, 2), "kernel_median_us": round(k_med_ms * 1e3, 2),
-                     "algorithmic_flop": flops, "hbm_side_GBps": round(algo_bytes / (k_avg_ms * 1e-3) / 1e9, 1)},
+                     "algorithmic_flop": flops, "hbm_side_GBps": round(algo_bytes / (k_avg_ms * 1e-3) / 1e9, 1),
+                     "sustained_mfma_tflops": sus_tf, "frac_of_sustained": round(achieved / sus_tf, 4),
+                     "sustained_mfma_clock_mhz": sus_mhz},
         "uncompressed_flash_decode_us": None if comp is None else comp["us"],
         "uncompressed_flash_decode_step_us": None if comp is None else comp["step_us"],
         "distinct_value_basis": distinct,
@@ -381,7 +459,7 @@ def bench_c2(args, dev):
         "config": {"workload": "c2 qAB_no_pe scores: batch 8, 32q/8kv, d128, L16384, rank 512, bf16 in / fp32 out", "kv_splits": S,
                    "buffers_rotated": nbuf},
         "roofline": {"bound": "hbm", "kernel": "latent_ring_kernel(scores)", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None if args.splits else C2_RING_HBM_BYTES,
+                     "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None if args.splits else recorded_traffic("c2"),
                      "kernel_avg_us": round(k_avg_ms * 1e3, 2), "kernel_median_us": round(k_med_ms * 1e3, 2),
                      "kernel_avg_us_one_buffer": round(warm_avg_ms * 1e3, 2), "algorithmic_bytes": algo_bytes},
         "parity_vs_oracle": parity,
@@ -426,7 +504,7 @@ def bench_c5(args, dev):
         "config": {"workload": "c5 MLA absorbed decode: batch 64, 16 heads, latent 512 + rope 64, ctx 8192, bf16", "kv_splits": S,
                    "buffers_rotated": nbuf},
         "roofline": {"bound": "hbm", "kernel": "latent_ring_kernel", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None if args.splits else C5_RING_HBM_BYTES,
+                     "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None if args.splits else recorded_traffic("c5"),
                      "kernel_avg_us": round(k_avg_ms * 1e3, 2), "kernel_median_us": round(k_med_ms * 1e3, 2),
                      "algorithmic_bytes": algo_bytes, "mfma_TFLOPs": round(flops / (k_avg_ms * 1e-3) / 1e12, 1)},
         "parity_vs_oracle": parity,
@@ -517,7 +595,7 @@ def bench_c4(args, dev, vfact):
         "roofline": {"bound": "hbm", "kernel": "latent_ring_kernel",
                      "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
-                     "traffic": C4_RING_HBM_BYTES if (not vfact and split == 4096) else None,
+                     "traffic": recorded_traffic("c4") if (not vfact and split == 4096) else None,
                      "note": "whole call (stage 1 + merge) over algorithmic bytes", "algorithmic_bytes": algo_bytes},
         "caller_splits_as_they_are_us": round(asis_ms * 1e3 / args.steps, 2),
         "parity_vs_oracle": parity,
@@ -628,7 +706,7 @@ def bench_ropedecode(args, dev):
         "ms_per_step": total_ms / args.steps, "step_us": step_q,
         "config": {"workload": "fused RoPE xKV decode, separate bases: batch 1, 32q/8kv, d128, kv_len %d, K rank %d, V rank %d, bf16"
                                % (L, rk, rv), "kv_splits": S},
-        "roofline": {"bound": "mfma", "kernel": "recon_fast_kernel (scores) + latent_ring_kernel (given scores), two passes", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": "recon_spec_kernel (scores) + latent_ring_kernel (given scores), two passes", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
                      "note": "whole call (pack, stage 1, merge) over algorithmic FLOP", "algorithmic_flop": flops,
                      "hbm_side_GBps": round(B * L * (rk + rv) * 2 / (us * 1e-6) / 1e9, 1)},
@@ -699,6 +777,8 @@ def main():
     ap.add_argument("--settle", type=float, default=1.5,
                     help="seconds of untimed calls of a workload before each of its measurements (the device reaches the clock "
                          "it sustains under that load); reported as settle_s")
+    ap.add_argument("--traffic-line", nargs=2, metavar=("WORKLOAD", "BYTES"),
+                    help="print the line of profiles/hbm_traffic_table.txt for a workload's measured HBM bytes and exit")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-comparator", action="store_true")
     ap.add_argument("--headline-first", action="store_true",
@@ -708,6 +788,9 @@ def main():
                     help="also run 3 plain device copies of 512 MiB (a kernel of known traffic, for scaling rocprof's "
                          "FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
+    if args.traffic_line:
+        print(traffic_line(args.traffic_line[0], int(float(args.traffic_line[1]))))
+        return
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
     from kernel_collections_amd import _lib

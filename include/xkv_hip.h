@@ -171,9 +171,10 @@ int xkv_softmax_pv_stage1(const float* scores, xkv_kv_operand V, float* partial,
  * Envelope: head_dim == 128, G = hq/hkv <= 16, rank % 32 == 0, rank <= 512, vA.dim % 64 == 0 <= 512.
  * With computed angles (sin_cos == NULL), G <= 8 and a workspace of xkv_recon_workspace_bytes() the call runs a
  * specialised kernel (kB packed once into the workspace, stationary in registers; v_mfma_f32_32x32x16; direct-to-LDS tile
- * rings): at ranks 256 / 384 / 512 with scores_out or vA the same tensor as kA the 4-wave kernel (2 x 2 rank/feature
- * wave split); at those ranks with a separate vA of rank 256 / 384 / 512 the 8-wave kernel (2 x 4 split, second row
- * stream for vA).  Otherwise the generic one.
+ * rings): at ranks 256 / 384 / 512 with scores_out or vA the same tensor as kA the wave-specialised kernel (four
+ * reconstruction waves in a 2 x 2 rank/feature split hand fp16 key tiles to four waves that rotate, score, soften and
+ * accumulate P.A; scores only at rank 256: the 4-wave form, two workgroups per CU); at those ranks with a separate vA of
+ * rank 256 / 384 / 512 the 8-wave kernel (2 x 4 split, second row stream for vA).  Otherwise the generic one.
  * Replaces _qAB_fwd[grid] at flash_recontruction/qAB/v1.py:135-145 (v3.py / v4.py / ref.py twins) and
  * _qAB_fwd_precomp[grid] at qAB/v2.py:170-186 in scores_out mode; the fused form has no single
  * reference launch - it composes that reconstruction with the stage 1 of

@@ -43,8 +43,8 @@ def _scores(q, Ak, Bk, inv_freq, sin_cos, pos_offset, sm_scale, out_dtype):
     Ak = ops.as_rows(Ak)
     Bk = Bk if Bk.stride(-1) == 1 else Bk.contiguous()
     out = torch.empty((bsz, num_heads, 1, kv_len), dtype=out_dtype, device=q.device)
-    # ranks 256 / 384 / 512 run the 4-wave MFMA kernel: one workgroup per CU above rank 256, two at rank 256 (its
-    # scores-only form fits twice: 252 registers, 78 KB of LDS); below, the register-staged scores kernel keeps 2-3
+    # ranks 384 / 512 run the wave-specialised MFMA kernel, one workgroup per CU; rank 256 the 4-wave kernel, whose scores-only
+    # form fits a CU twice (252 registers, 78 KB of LDS); below, the register-staged scores kernel keeps 2-3
     n_splits = ops.occupancy_splits(bsz, num_kv_heads, kv_len, tile=32, waves=1 if rank > 256 else (2 if rank > 128 else 3))
     splits = ops.uniform_splits(bsz, n_splits, q.device)
     ops.recon_stage1(q3, Ak, Bk, None, None, None, out, splits, None, bsz, num_heads, num_kv_heads, kv_len,
