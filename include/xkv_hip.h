@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define XKV_ABI_VERSION 5
+#define XKV_ABI_VERSION 6
 
 enum { XKV_F16 = 0, XKV_BF16 = 1, XKV_F32 = 2 };
 
@@ -266,6 +266,14 @@ int xkv_plan_splits(const int32_t* kv_lens, const int32_t* num_kv_splits, int ba
  *   (to_lds == 2: workgroups * 256 floats, the number of 16-byte packets each thread handed on). */
 int xkv_ceiling_mfma(float* out, int workgroups, int iters, int dtype, void* stream);
 int xkv_ceiling_stream(const void* src, int64_t bytes, int workgroups, int to_lds, int depth, float* out, void* stream);
+
+/* Test aid (no counterpart in the reference; tests/test_gpu_lds_poison.py).  The LDS is not cleared between kernels.  With
+ * seen == NULL: fills all 160 KiB of LDS of every CU with `pattern` (0x7FFF7FFF is a NaN as fp16, bf16 and fp32), so that a
+ * kernel launched next on the stream which reads LDS that it has not written yet, or whose asynchronous tile loads have not
+ * landed, computes NaNs instead of plausible stale rows.  With seen != NULL (2 int32, zeroed by the caller): one workgroup
+ * per CU adds the number of LDS words that still hold `pattern` to seen[0] and the number it looked at to seen[1], which tells
+ * a test whether the poison of the previous call was still there. */
+int xkv_poison_lds(uint32_t pattern, int32_t* seen, void* stream);
 
 #ifdef __cplusplus
 }

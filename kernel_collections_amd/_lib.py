@@ -12,12 +12,13 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("XKV_HIP_LIB", os.path.join(_HERE, "libxkv_hip.so"))  # override: another build of the same ABI
 
 XKV_F16, XKV_BF16, XKV_F32 = 0, 1, 2
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 EXPORTS = (
     "xkv_abi_version", "xkv_error_string", "xkv_rope_table", "xkv_absorb_q",
     "xkv_blockdiag_q", "xkv_latent_stage1", "xkv_recon_stage1", "xkv_recon_workspace_bytes", "xkv_merge_stage2",
     "xkv_recon_stage1_static", "xkv_rope_apply", "xkv_ceiling_mfma", "xkv_ceiling_stream", "xkv_plan_splits", "xkv_softmax_pv_stage1",
+    "xkv_poison_lds",
 )
 STATIC_SCRATCH_BYTES = 4 << 20
 XKV_ESCRATCH = -5
@@ -75,6 +76,8 @@ def _declare(lib):
     lib.xkv_softmax_pv_stage1.restype = c_int
     lib.xkv_softmax_pv_stage1.argtypes = [c_void_p, KVOperand, c_void_p, c_void_p, c_void_p, c_void_p,
                                           c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p]
+    lib.xkv_poison_lds.restype = c_int
+    lib.xkv_poison_lds.argtypes = [ctypes.c_uint32, c_void_p, c_void_p]
     lib.xkv_plan_splits.restype = c_int
     lib.xkv_plan_splits.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]
 

@@ -1,4 +1,4 @@
-// Two measurement aids, not part of the decode path: what this GPU sustains with NOTHING but the instruction a
+// Measurement and test aids, not part of the decode path.  Two ceilings: what this GPU sustains with NOTHING but the instruction a
 // kernel is bound by.  (1) v_mfma_f32_32x32x16 on register operands, every wave of every CU; (2) an HBM read
 // stream, into registers or straight into LDS (global_load_lds_dwordx4), with no use of the data.  The scan and
 // reconstruction kernels are judged against the published peaks; these two figures say how much of the distance
@@ -135,6 +135,45 @@ static int launch_stream(const void* src, int64_t bytes, int wgs, float* out, hi
 }  // namespace xkv
 
 using namespace xkv;
+
+// ---- (3) a test aid: LDS is not cleared between kernels, so a kernel that reads a part of its LDS before anything of its own
+// has landed there computes on whatever the previous kernel on that CU left.  poison_lds_kernel leaves a pattern that is a NaN
+// as fp16, bf16 and fp32 in all 160 KiB of every CU (one workgroup fills a CU's LDS, so no two of them share one; four per CU
+// so that every CU gets one), and count_lds_kernel reports how much of a fresh workgroup's LDS still holds it.
+constexpr int POISON_LDS_BYTES = 160 * 1024;
+__global__ __launch_bounds__(1024) void poison_lds_kernel(unsigned pattern) {
+  extern __shared__ __attribute__((aligned(16))) unsigned lds_words[];
+  for (int i = threadIdx.x; i < POISON_LDS_BYTES / 4; i += 1024) lds_words[i] = pattern;
+  __syncthreads();
+  const unsigned back = lds_words[(threadIdx.x * 37) % (POISON_LDS_BYTES / 4)];
+  asm volatile("" ::"v"(back));   // a use of the LDS contents: keeps the stores alive
+}
+__global__ __launch_bounds__(1024) void count_lds_kernel(unsigned pattern, int32_t* __restrict__ seen) {
+  extern __shared__ __attribute__((aligned(16))) unsigned lds_words[];
+  int n = 0;
+  for (int i = threadIdx.x; i < POISON_LDS_BYTES / 4; i += 1024) n += lds_words[i] == pattern;
+  atomicAdd(&seen[0], n);
+  if (threadIdx.x == 0) atomicAdd(&seen[1], POISON_LDS_BYTES / 4);
+}
+
+extern "C" int xkv_poison_lds(uint32_t pattern, int32_t* seen, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  int dev = 0, cus = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e != hipSuccess) return (int)e;
+  static DynLds lds[2];
+  if (!seen) {
+    const int rc = ensure_dynamic_lds(lds[0], reinterpret_cast<const void*>(poison_lds_kernel), POISON_LDS_BYTES);
+    if (rc != XKV_OK) return rc;
+    poison_lds_kernel<<<dim3(4 * cus), dim3(1024), POISON_LDS_BYTES, st>>>(pattern);
+  } else {
+    const int rc = ensure_dynamic_lds(lds[1], reinterpret_cast<const void*>(count_lds_kernel), POISON_LDS_BYTES);
+    if (rc != XKV_OK) return rc;
+    count_lds_kernel<<<dim3(cus), dim3(1024), POISON_LDS_BYTES, st>>>(pattern, seen);
+  }
+  return launch_status();
+}
 
 extern "C" int xkv_ceiling_mfma(float* out, int workgroups, int iters, int dtype, void* stream) {
   if (!out || workgroups <= 0 || iters <= 0) return XKV_EINVAL;

@@ -13,7 +13,7 @@ _xkv.xkv_recon_stage1.restype = c_int
 _xkv.xkv_recon_stage1.argtypes = [c_void_p, KVOperand, c_void_p, c_int64, c_int64, c_int64, KVOperand,
     c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
     c_float, c_int, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int, c_void_p]
-assert _xkv.xkv_abi_version() == 5
+assert _xkv.xkv_abi_version() == 6
 
 def qAB(q, A, B, theta=1e7):                       # same signature as flash_recontruction/qAB/v1.py:90
     bsz, hq, _, d = q.shape; L, r = A.shape[1], A.shape[2]; hkv = B.shape[1]
