@@ -109,7 +109,8 @@ def test_qab_nope_shared_factor_stride0_and_row_strides(dev):
 @pytest.mark.parametrize("b,hq,hkv,L,r,theta", [(2, 32, 8, 1000, 512, 5e5), (1, 8, 2, 77, 256, 1e7),
                                                 (1, 16, 1, 2085, 384, 1e4), (2, 4, 4, 40, 192, 1e7),
                                                 (2, 8, 2, 300, 384, 5e5),    # wave-specialised kernel at rank 384, scores mode
-                                                (1, 16, 2, 1500, 256, 1e7)])  # ... at rank 256, 8 heads per kv head
+                                                (1, 16, 2, 1500, 256, 1e7),   # ... at rank 256, 8 heads per kv head
+                                                (1, 48, 8, 700, 512, 5e5), (2, 15, 3, 333, 384, 1e4)])  # 6 and 5 heads per kv head
 def test_qab_rope(dev, dtype, b, hq, hkv, L, r, theta):
     d = 128
     q, A, B = gen((b, hq, 1, d), std=0.5, dtype=dtype, seed=1), gen((b, L, r), dtype=dtype, seed=2), \
@@ -217,7 +218,10 @@ def test_fused_rope(dev, dtype, b, hq, hkv, L, rk, rv, S, shared):
     (2, 32, 8, 384, 384, True, [900, 1200], 4, 0),
     (2, 16, 4, 256, 256, True, [33, 4000], 6, 131072 - 4000),
     (1, 16, 2, 384, 384, True, [1500], 3, 0),              # the wave-specialised kernel at ranks 384 / 256: 8 heads per kv head ...
-    (2, 8, 8, 256, 256, True, [100, 257], 2, 50000)])      # ... and one
+    (2, 8, 8, 256, 256, True, [100, 257], 2, 50000),       # ... and one
+    (1, 48, 8, 512, 512, True, [1100], 3, 0),              # 6 query heads per kv head: head slots 6 and 7 of the 8 are empty
+    (2, 40, 8, 384, 256, False, [70, 1300], 2, 7),         # 5 per kv head
+    (1, 21, 3, 256, 256, True, [999], 4, 0)])              # 7 per kv head, 3 kv heads
 @pytest.mark.parametrize("form", ["fused", "two_pass", "as_shipped"])
 def test_fused_rope_wide_kernels(dev, dtype, b, hq, hkv, rk, rv, shared, lens, S, off, form, monkeypatch):
     # a value basis of its own runs either fused (one kernel, two row streams) or as two passes (scores, then softmax + P.v_A);
