@@ -221,7 +221,10 @@ def test_fused_rope(dev, dtype, b, hq, hkv, L, rk, rv, S, shared):
     (2, 8, 8, 256, 256, True, [100, 257], 2, 50000),       # ... and one
     (1, 48, 8, 512, 512, True, [1100], 3, 0),              # 6 query heads per kv head: head slots 6 and 7 of the 8 are empty
     (2, 40, 8, 384, 256, False, [70, 1300], 2, 7),         # 5 per kv head
-    (1, 21, 3, 256, 256, True, [999], 4, 0)])              # 7 per kv head, 3 kv heads
+    (1, 21, 3, 256, 256, True, [999], 4, 0),               # 7 per kv head, 3 kv heads
+    (2, 32, 8, 512, 512, True, [1, 32], 2, 0),             # one token; exactly one tile (the second split is dead)
+    (2, 32, 8, 512, 512, True, [192, 193], 1, 31),         # exactly the six tiles of one unrolled block, and one token more
+    (2, 16, 4, 384, 384, False, [1, 191], 3, 0)])
 @pytest.mark.parametrize("form", ["fused", "two_pass", "as_shipped"])
 def test_fused_rope_wide_kernels(dev, dtype, b, hq, hkv, rk, rv, shared, lens, S, off, form, monkeypatch):
     # a value basis of its own runs either fused (one kernel, two row streams) or as two passes (scores, then softmax + P.v_A);
