@@ -328,12 +328,33 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
       }
       __syncthreads();
       const int n_here = (ngrp - base) < chunk ? (ngrp - base) : chunk;
-      for (int idx = threadIdx.x; idx < 4 * d_out; idx += blockDim.x) {
-        const int gi = idx / d_out, c = idx - gi * d_out;
-        if (g0 + gi < G) {
-          float sacc = 0.f;
-          for (int k = 0; k < n_here; ++k) sacc += red[(k * 4 + gi) * cols + c];
-          fin[idx] = (base == 0 ? 0.f : fin[idx]) + sacc;
+      const int nout = 4 * d_out;
+      if (nout <= 128 && ngrp <= chunk) {
+        // a narrow column block: fewer totals than threads and many rank groups (one pass).  256 / nout threads share a total's
+        // groups, so that nobody walks 64 LDS words one after the other; their sums meet in `fin`.
+        const int parts = 256 / nout, o = threadIdx.x % nout, part = threadIdx.x / nout;
+        const int gi = o / d_out, c = o - gi * d_out;
+        float sacc = 0.f;
+        if (part < parts) {
+#pragma unroll 8
+          for (int k = part; k < n_here; k += parts) sacc += red[(k * 4 + gi) * cols + c];
+          fin[part * nout + o] = sacc;
+        }
+        __syncthreads();
+        if (threadIdx.x < nout) {
+          float tot = fin[threadIdx.x];
+          for (int q = 1; q < parts; ++q) tot += fin[q * nout + threadIdx.x];
+          fin[threadIdx.x] = tot;
+        }
+      } else {
+        for (int idx = threadIdx.x; idx < nout; idx += blockDim.x) {
+          const int gi = idx / d_out, c = idx - gi * d_out;
+          if (g0 + gi < G) {
+            float sacc = 0.f;
+#pragma unroll 8
+            for (int k = 0; k < n_here; ++k) sacc += red[(k * 4 + gi) * cols + c];
+            fin[idx] = (base == 0 ? 0.f : fin[idx]) + sacc;
+          }
         }
       }
     }
@@ -365,6 +386,7 @@ static int launch_merge(const float* partial, const float* lse, void* out, const
   const int g = hq / hkv;
   const bool enough_wgs = vB && (int64_t)hkv * batch >= 128;   // vB costs more than the partial rows: keep it read once per kv head
   int hpw = (g > 16 || (max_splits > 16 && !enough_wgs)) ? 1 : g;
+  if (!vB) hpw = 1;   // nothing is shared by the heads of a kv head without an up-projection: one workgroup per head
   // dynamic LDS beside the kernel's 8 KiB of static LDS: the default limit of 64 KiB per workgroup must hold both; a group
   // of heads that does not fit is merged one head per workgroup, and a single head that does not fit is refused
   constexpr size_t LDS_LIMIT = 64 * 1024, STATIC_LDS = 8 * 1024;
@@ -378,6 +400,10 @@ static int launch_merge(const float* partial, const float* lse, void* out, const
   // over more workgroups
   int zb = 1;
   if (vB && (hq / hpw) * batch < 128 && max_splits >= 64 && d_out % 32 == 0) zb = d_out >= 512 ? 4 : d_out >= 256 ? 2 : 1;
+  // few splits: the merge itself is cheap to repeat, and what is left is the latency of the vB rows a thread reads one after
+  // the other - column blocks of >= 32 until the grid has 512 workgroups (a thread then reads dv / 64 rows instead of dv / 16)
+  if (vB && max_splits <= 16)
+    while ((int64_t)(hq / hpw) * batch * zb < 512 && d_out % (zb * 2 * 8) == 0 && d_out / (zb * 2) >= 32) zb *= 2;
   merge_stage2_kernel<O, TB><<<dim3(hq / hpw, batch, zb), dim3(256), shm, st>>>(partial, lse, (O*)out, (const TB*)vB, sVb, sVh,
                                                                                sVr, d_out, ns, kl, hq, hkv, kv_len, max_splits,
                                                                                dv, sOb, sOh, hpw, lse_out, sLb, sLh, d_out / zb, split_cap, split_plan);
