@@ -170,6 +170,7 @@ __global__ __launch_bounds__(256) void blockdiag_q_kernel(const T* __restrict__ 
 // (reference order: increasing split id, running max of lse), then optionally multiplies the
 // merged rank-space rows by vB[b, kh] (read once for the G heads).
 // ----------------------------------------------------------------------------------------------
+constexpr int MERGE_RED_FLOATS = 32 * 4 * 64, MERGE_FIN_FLOATS = 4 * 512;   // the kernel's static LDS (the launcher counts it)
 template <typename O, typename TB>
 __global__ __launch_bounds__(256) void merge_stage2_kernel(
     const float* __restrict__ partial, const float* __restrict__ lse, O* __restrict__ out,
@@ -178,7 +179,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     int hq, int hkv, int kv_len, int max_splits, int dv, int64_t sOb, int64_t sOh, int hpw,
     float* __restrict__ lse_out, int64_t sLb, int64_t sLh, int d_blk, int split_cap, const int32_t* __restrict__ split_plan) {
   extern __shared__ float merged[];  // [G][dv], then the split weights [G][max_splits]
-  __shared__ float fin[4 * 512];     // per-head-block totals of the up-projection
+  __shared__ float fin[MERGE_FIN_FLOATS];     // per-head-block totals of the up-projection
   // this workgroup: heads hfirst .. hfirst + G - 1 of sequence b, all of kv head kh (G = hpw divides the GQA group size)
   const int G = hpw, hfirst = blockIdx.x * hpw, kh = hfirst / (hq / hkv), b = blockIdx.y;
   // blockIdx.z: a block of d_blk output columns of the up-projection (every block repeats the merge: when the grid is
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
   // loads of vB, several in flight, then a reduction over the rank groups through LDS.
   typedef typename Elem<TB>::vec8 vec8;
   const TB* Bh = vB + b * sVb + kh * sVh;
-  __shared__ float red[32 * 4 * 64];                 // [rank group][4 heads][columns of the block]  (<= 32 KiB)
+  __shared__ float red[MERGE_RED_FLOATS];            // [rank group][4 heads][columns of the block]: 32 KiB
   const int ncb = (d_out + 7) >> 3;                  // 8-column blocks (d_out <= 512 -> <= 64)
   const int ngrp = 256 / ncb;                        // rank groups
   const int cb = threadIdx.x % ncb, grp = threadIdx.x / ncb;
@@ -317,14 +318,15 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
     }
     // reduce over the rank groups through LDS, `chunk` groups per pass (as many as fit `red`)
     const int cols = ncb * 8;                        // <= 512
-    const int chunk = 32 * 64 / cols;                // >= 4
+    const int gstride = 4 * cols;                    // a rank group's 4 x cols floats
+    const int chunk = MERGE_RED_FLOATS / gstride;    // groups per pass (>= 4): what fits `red`
     for (int base = 0; base < ngrp; base += chunk) {
       __syncthreads();
       if (active && grp >= base && grp < base + chunk) {
 #pragma unroll
         for (int gi = 0; gi < 4; ++gi)
 #pragma unroll
-          for (int e = 0; e < 8; ++e) red[((grp - base) * 4 + gi) * cols + cb * 8 + e] = acc[gi][e];
+          for (int e = 0; e < 8; ++e) red[(grp - base) * gstride + gi * cols + cb * 8 + e] = acc[gi][e];
       }
       __syncthreads();
       const int n_here = (ngrp - base) < chunk ? (ngrp - base) : chunk;
@@ -337,7 +339,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
         float sacc = 0.f;
         if (part < parts) {
 #pragma unroll 8
-          for (int k = part; k < n_here; k += parts) sacc += red[(k * 4 + gi) * cols + c];
+          for (int k = part; k < n_here; k += parts) sacc += red[k * gstride + gi * cols + c];
           fin[part * nout + o] = sacc;
         }
         __syncthreads();
@@ -352,7 +354,7 @@ __global__ __launch_bounds__(256) void merge_stage2_kernel(
           if (g0 + gi < G) {
             float sacc = 0.f;
 #pragma unroll 8
-            for (int k = 0; k < n_here; ++k) sacc += red[(k * 4 + gi) * cols + c];
+            for (int k = 0; k < n_here; ++k) sacc += red[k * gstride + gi * cols + c];
             fin[idx] = (base == 0 ? 0.f : fin[idx]) + sacc;
           }
         }
@@ -387,15 +389,14 @@ static int launch_merge(const float* partial, const float* lse, void* out, const
   const bool enough_wgs = vB && (int64_t)hkv * batch >= 128;   // vB costs more than the partial rows: keep it read once per kv head
   int hpw = (g > 16 || (max_splits > 16 && !enough_wgs)) ? 1 : g;
   if (!vB) hpw = 1;   // nothing is shared by the heads of a kv head without an up-projection: one workgroup per head
-  // dynamic LDS beside the kernel's 8 KiB of static LDS: the default limit of 64 KiB per workgroup must hold both; a group
-  // of heads that does not fit is merged one head per workgroup, and a single head that does not fit is refused
-  constexpr size_t LDS_LIMIT = 64 * 1024, STATIC_LDS = 8 * 1024;
-  size_t shm = (size_t)hpw * (dv + max_splits) * sizeof(float);
-  if (shm + STATIC_LDS > LDS_LIMIT) {
-    hpw = 1;
-    shm = (size_t)(dv + max_splits) * sizeof(float);
-    if (shm + STATIC_LDS > LDS_LIMIT) return XKV_EUNSUPPORTED;
-  }
+  // dynamic LDS beside the kernel's static LDS (the up-projection's reduction buffers): the default limit of 64 KiB per
+  // workgroup must hold both; a group of heads that does not fit is merged one head per workgroup, and a single head that
+  // does not fit is refused
+  constexpr size_t LDS_LIMIT = 64 * 1024, STATIC_LDS = (MERGE_RED_FLOATS + MERGE_FIN_FLOATS) * sizeof(float);
+  auto dyn_lds = [&](int heads) { return (size_t)heads * (dv + max_splits) * sizeof(float); };
+  while (hpw > 1 && (g % hpw != 0 || dyn_lds(hpw) + STATIC_LDS > LDS_LIMIT)) --hpw;   // the largest group of heads that fits
+  const size_t shm = dyn_lds(hpw);
+  if (shm + STATIC_LDS > LDS_LIMIT) return XKV_EUNSUPPORTED;
   // a small grid over many splits is bound by the latency of its partial-row loads: split the up-projection's columns
   // over more workgroups
   int zb = 1;

@@ -53,7 +53,7 @@ def test_argument_errors_are_reported_before_any_launch():
                                    ctypes.c_void_p(16), 0, null, 0, _lib.XKV_BF16, null)
     assert rc == _lib.XKV_ESCRATCH and b"static device array" in L.xkv_error_string(rc)
     # the merge keeps one head's merged row and split weights in the LDS: a split count that cannot fit beside the kernel's
-    # static 8 KiB is refused before any launch (512 + 14000 floats > 56 KiB)
+    # static buffers is refused before any launch (512 + 14000 floats = 58 KB of the 64 KiB a workgroup may have)
     rc = L.xkv_merge_stage2(ctypes.c_void_p(16), ctypes.c_void_p(16), ctypes.c_void_p(16), null, 0, 0, 0, 0, _lib.XKV_BF16,
                             ns, null, 1, 8, 1, 14000 * 32, 14000, 0, null, 512, 8 * 512, 512, _lib.XKV_F32, null, 0, 0, null)
     assert rc == -2
