@@ -79,3 +79,56 @@ def test_static_scratch_rejects_what_does_not_fit(dev):
     assert _lib.lib().xkv_recon_workspace_bytes(b, hkv, r, c_int64(kB.stride(0))) > _lib.STATIC_SCRATCH_BYTES
     with pytest.raises(RuntimeError, match="static device array"):
         _call(True, q, kA, kB, kA, 1, 5e5, dev)
+
+
+def test_static_scratch_entry_point_under_graph_capture(dev):
+    """What the entry point is for: after one warm-up call per shape it can be recorded into a HIP graph (nothing in it
+    allocates, looks up symbols or sets attributes any more).  The graph - stage 1 into fixed workspaces, then the merge - is
+    replayed three times with new queries in the captured input buffer, with eager work and synchronisations between the
+    replays, and every replay is compared with the eager result for the same query."""
+    dtype, theta = torch.bfloat16, 5e5
+    b, hq, hkv, L, r, S, d = 2, 32, 8, 1500, 512, 3, 128
+    kA = gen((b, L, r), dtype=dtype, seed=51).to(dev)
+    kB = gen((1, hkv, r, d), std=r ** -0.5, dtype=dtype, seed=52).to(dev).expand(b, -1, -1, -1)
+    vB = gen((1, hkv, r, d), std=r ** -0.5, dtype=dtype, seed=53).to(dev).expand(b, -1, -1, -1)
+    q_in = torch.zeros((b, hq, d), dtype=dtype, device=dev)
+    partial = torch.zeros((b, hq, S, r), device=dev)
+    lse = torch.zeros((b, hq, S), device=dev)
+    out = torch.zeros((b, hq, d), dtype=dtype, device=dev)
+    ns = ops.uniform_splits(b, S, dev)
+    inv = ops.rope_inv_freq(d, theta, dev)
+    lib = _lib.lib()
+
+    def step():
+        a_op = kv_operand(kA, kA.stride(0), kA.stride(1), 0, r)
+        rc = lib.xkv_recon_stage1_static(ptr(q_in), a_op, ptr(kB), c_int64(kB.stride(0)), c_int64(kB.stride(1)),
+                                         c_int64(kB.stride(2)), a_op, ptr(partial), ptr(lse), ptr(None), 0, ptr(ns), ptr(None),
+                                         b, hq, hkv, L, S, c_float(d ** -0.5), 1, ptr(inv), c_int64(0), ptr(None), c_int64(0),
+                                         dtype_code(dtype), stream_ptr(q_in))
+        _lib.check(rc, "stage 1")
+        ops.merge_stage2(partial, lse, out, vB, ns, None, b, hq, hkv, L, S)
+
+    queries = [gen((b, hq, d), std=0.5, dtype=dtype, seed=60 + i).to(dev) for i in range(4)]
+    q_in.copy_(queries[0])
+    step()                                   # warm-up of this shape, outside the capture
+    torch.cuda.synchronize()
+    eager = []
+    for qq in queries:
+        q_in.copy_(qq)
+        step()
+        eager.append(out.clone())
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        q_in.copy_(queries[0])
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.synchronize()
+    for i in (1, 2, 3):
+        q_in.copy_(queries[i])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager[i]), f"replay {i} differs from the eager call"
+        scratch = torch.randn(1 << 16, device=dev).sum().item()   # eager work between the replays
+        assert scratch == scratch
