@@ -144,7 +144,8 @@ def test_qab_rope_long_positions(dev):
 @pytest.mark.parametrize("b,hq,hkv,L,rk,rv,S", [(2, 32, 8, 3000, 256, 384, 8), (1, 32, 8, 700, 512, 512, 3),
                                                 (3, 8, 8, 129, 192, 64, 2), (1, 16, 4, 4096, 384, 256, 16),
                                                 (2, 32, 8, 40, 512, 512, 2), (1, 8, 2, 3, 512, 512, 4),   # fewer live splits than asked
-                                                (2, 16, 8, 1000, 384, 256, 4), (1, 8, 8, 777, 512, 256, 3)])
+                                                (2, 16, 8, 1000, 384, 256, 4), (1, 8, 8, 777, 512, 256, 3),
+                                                (1, 128, 8, 600, 512, 512, 2)])   # 16 heads per kv head: the merge's head groups
 def test_fused_nope(dev, dtype, b, hq, hkv, L, rk, rv, S):
     d = 128
     q = gen((b, hq, d), std=1 / 3, dtype=dtype, seed=1)
